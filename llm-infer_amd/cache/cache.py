@@ -62,7 +62,7 @@ class KVGroup:
     def __init__(self, spec: KVSpec, entries, n_slots, n_pages, max_positions, dtype, device, round_to=None):
         self.spec, self.entries, self.round_to = spec, list(entries), round_to
         self.k_elems = spec.n_kv_heads * PAGE * spec.head_dim
-        self.v_elems = spec.n_kv_heads * PAGE * _round_up(spec.head_dim, 32)
+        self.v_elems = spec.n_kv_heads * PAGE * _round_up(spec.v_head_dim or spec.head_dim, 32)
         self.layer_elems = self.k_elems + self.v_elems
         self.page_elems = self.layer_elems * len(self.entries)
         self.n_pages = n_pages

@@ -7,10 +7,12 @@ from dataclasses import dataclass
 
 @dataclass(frozen=True)
 class KVSpec:
-    """Keys and values for every token (``window`` None) or for the last ``window`` tokens."""
+    """Keys and values for every token (``window`` None) or for the last ``window`` tokens.
+    ``v_head_dim`` None: values have the keys' head size."""
     n_kv_heads: int
     head_dim: int
     window: int | None = None
+    v_head_dim: int | None = None
 
 
 @dataclass(frozen=True)

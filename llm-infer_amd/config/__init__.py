@@ -1,4 +1,5 @@
 from .spec import PartSpec, SubLayerSpec, LayerSpec, ScheduleEntry, ModelSpec, ConfigError
 from .llama import LlamaConfig
+from .manirax import ManiraxConfig
 
-__all__ = ["PartSpec", "SubLayerSpec", "LayerSpec", "ScheduleEntry", "ModelSpec", "ConfigError", "LlamaConfig"]
+__all__ = ["PartSpec", "SubLayerSpec", "LayerSpec", "ScheduleEntry", "ModelSpec", "ConfigError", "LlamaConfig", "ManiraxConfig"]

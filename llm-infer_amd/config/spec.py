@@ -46,6 +46,7 @@ class LayerSpec:
     block: str
     sublayers: tuple
     position: PartSpec | None = None
+    block_params: dict = field(default_factory=dict)      # constants of the arrangement (a residual scale, say)
 
     @classmethod
     def mixer_then_feed_forward(cls, block: str, mixer: PartSpec, feed_forward: PartSpec, mixer_norm: PartSpec,
@@ -67,7 +68,7 @@ class ScheduleEntry:
 class ModelSpec:
     hidden_size: int
     vocab_size: int
-    max_positions: int
+    max_positions: int            # 0: the design sets no bound (the engine then takes what its cache holds)
     embedding: PartSpec
     layers: tuple
     schedule: tuple

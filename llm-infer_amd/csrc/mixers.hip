@@ -1,0 +1,490 @@
+// Kernels of the mixers and arrangements beside the softmax decoder's: layer norm (alone, and fused with
+// the scaled residual sum of a post-norm layer), token shift with its per-sequence state, rotation in the
+// half layout followed by a unit-RMS norm of q and k with the write into the paged cache, attention whose
+// weights are sigmoids of the scores, linear attention with a constant decay per head and a float32 state
+// per sequence, the gated RMS norm behind it, and the PolyNorm activation.  Every size is a run-time value.
+// Whatever a norm, a score, an attention weight or a recurrent state is made of is float32 here, whatever
+// the type of the matrices.
+#include "common.h"
+
+struct Pages {
+    const void* k;
+    const void* v;
+    int64_t page_stride;            // elements from one page to the next
+    const int* page_table;          // [slots, max_pages]
+    int max_pages;
+};
+
+__device__ __forceinline__ float sigmoidf(float z) { return 1.f / (1.f + expf(-z)); }
+__device__ __forceinline__ float siluf(float z) { return z / (1.f + expf(-z)); }
+
+// ---------------------------------------------------------------------------
+// Layer norm with a weight and no bias: out = (x - mean) / sqrt(var + eps) * w, var the mean of the
+// squared deviations.  `rows` (may be null) picks rows.
+// ---------------------------------------------------------------------------
+template <class TO>
+__global__ void layernorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                 const int* __restrict__ rows, TO* __restrict__ out, int d, float eps) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const float* xr = x + (int64_t)(rows ? rows[r] : r) * d;
+    TO* o = out + (int64_t)r * d;
+    float s = 0.f;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) s += xr[i];
+    const float mean = block_sum(s, scratch) / (float)d;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) { const float v = xr[i] - mean; ss += v * v; }
+    const float sd = sqrtf(block_sum(ss, scratch) / (float)d + eps);
+    for (int i = threadIdx.x; i < d; i += blockDim.x) o[i] = from_f32<TO>((xr[i] - mean) / sd * w[i]);
+}
+
+extern "C" int li_layernorm(const float* x, const float* w, const int* rows, void* out, int out_dt, int n_rows,
+                            int d, float eps, hipStream_t stream) {
+    if (n_rows <= 0) return LI_OK;
+    if (d <= 0) return LI_BAD_ARG;
+    dim3 grid(n_rows), block(d >= 2048 ? 512 : (d >= 256 ? 256 : 64));
+    if (out_dt == DT_F32) layernorm_kernel<float><<<grid, block, 0, stream>>>(x, w, rows, (float*)out, d, eps);
+    else if (out_dt == DT_F16) layernorm_kernel<f16><<<grid, block, 0, stream>>>(x, w, rows, (f16*)out, d, eps);
+    else if (out_dt == DT_BF16) layernorm_kernel<bf16><<<grid, block, 0, stream>>>(x, w, rows, (bf16*)out, d, eps);
+    else return LI_BAD_ARG;
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// The residual step of a layer whose norm comes after the sum:
+//   x <- LN(alpha * x + (s1 * y1 + s2 * y2)) * w        (y2 may be null)
+// in place on the float32 rows of x; `copy` (may be null) receives the new rows in a 16-bit type as well,
+// for the product that reads them next.
+// ---------------------------------------------------------------------------
+template <class TC>
+__global__ void add_layernorm_kernel(float* __restrict__ x, float alpha, const float* __restrict__ y1, float s1,
+                                     const float* __restrict__ y2, float s2, const float* __restrict__ w, float eps,
+                                     TC* __restrict__ copy, int d) {
+    __shared__ float scratch[16];
+    const int64_t base = (int64_t)blockIdx.x * d;
+    float* xr = x + base;
+    float s = 0.f;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+        float y = s1 * y1[base + i];
+        if (y2) y += s2 * y2[base + i];
+        const float v = alpha * xr[i] + y;
+        xr[i] = v;                                // read back by the same thread below
+        s += v;
+    }
+    const float mean = block_sum(s, scratch) / (float)d;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) { const float v = xr[i] - mean; ss += v * v; }
+    const float sd = sqrtf(block_sum(ss, scratch) / (float)d + eps);
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+        const float v = (xr[i] - mean) / sd * w[i];
+        xr[i] = v;
+        if (copy) copy[base + i] = from_f32<TC>(v);
+    }
+}
+
+extern "C" int li_add_layernorm(float* x, float alpha, const float* y1, float s1, const float* y2, float s2,
+                                const float* w, float eps, void* copy, int copy_dt, int n_rows, int d,
+                                hipStream_t stream) {
+    if (n_rows <= 0) return LI_OK;
+    if (d <= 0 || !y1) return LI_BAD_ARG;
+    dim3 grid(n_rows), block(d >= 2048 ? 512 : (d >= 256 ? 256 : 64));
+    if (!copy || copy_dt == DT_F32)
+        add_layernorm_kernel<float><<<grid, block, 0, stream>>>(x, alpha, y1, s1, y2, s2, w, eps, (float*)copy, d);
+    else if (copy_dt == DT_F16)
+        add_layernorm_kernel<f16><<<grid, block, 0, stream>>>(x, alpha, y1, s1, y2, s2, w, eps, (f16*)copy, d);
+    else if (copy_dt == DT_BF16)
+        add_layernorm_kernel<bf16><<<grid, block, 0, stream>>>(x, alpha, y1, s1, y2, s2, w, eps, (bf16*)copy, d);
+    else return LI_BAD_ARG;
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// out = y1 * s1 (+ y2 * s2) added into x: the same sum for an arrangement without the norm behind it.
+__global__ void add_scaled_kernel(float* __restrict__ x, const float* __restrict__ y1, float s1,
+                                  const float* __restrict__ y2, float s2, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float y = s1 * y1[i];
+    if (y2) y += s2 * y2[i];
+    x[i] += y;
+}
+
+extern "C" int li_add_scaled(float* x, const float* y1, float s1, const float* y2, float s2, int64_t n,
+                             hipStream_t stream) {
+    if (n <= 0) return LI_OK;
+    add_scaled_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(x, y1, s1, y2, s2, n);
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// float32 -> a 16-bit type
+template <class TO>
+__global__ void cast_kernel(const float* __restrict__ x, TO* __restrict__ out, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = from_f32<TO>(x[i]);
+}
+
+extern "C" int li_cast(const float* x, void* out, int out_dt, int64_t n, hipStream_t stream) {
+    if (n <= 0) return LI_OK;
+    dim3 grid((unsigned)((n + 255) / 256)), block(256);
+    if (out_dt == DT_F16) cast_kernel<f16><<<grid, block, 0, stream>>>(x, (f16*)out, n);
+    else if (out_dt == DT_BF16) cast_kernel<bf16><<<grid, block, 0, stream>>>(x, (bf16*)out, n);
+    else return LI_BAD_ARG;
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Token shift: out_t = x_t + (x_{t-1} - x_t) * mu, channel by channel, where x_{t-1} is the row of the
+// token before in the same sequence: the row above in this step, or, for the first token that a sequence
+// brings to this step, the row that the step before left in `state[slot]`; zeros at position 0.  A second
+// kernel then leaves each sequence's last row of this step in its state.  The rows of one sequence are
+// consecutive and no two sequences share a slot, so a change of tok_slot marks a sequence's edge.
+// ---------------------------------------------------------------------------
+template <class TO>
+__global__ void token_shift_kernel(const float* __restrict__ x, const float* __restrict__ mu,
+                                   const float* __restrict__ state, const int* __restrict__ pos,
+                                   const int* __restrict__ tok_slot, TO* __restrict__ out, int d) {
+    const int t = blockIdx.x;
+    const int slot = tok_slot[t];
+    const bool first = t == 0 || tok_slot[t - 1] != slot;
+    const float* prev = pos[t] == 0 ? nullptr : (first ? state + (int64_t)slot * d : x + (int64_t)(t - 1) * d);
+    const float* xr = x + (int64_t)t * d;
+    TO* o = out + (int64_t)t * d;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+        const float h = xr[i], p = prev ? prev[i] : 0.f;
+        o[i] = from_f32<TO>(h + (p - h) * mu[i]);
+    }
+}
+
+__global__ void token_shift_save_kernel(const float* __restrict__ x, float* __restrict__ state,
+                                        const int* __restrict__ tok_slot, int d, int n_tokens) {
+    const int t = blockIdx.x;
+    const int slot = tok_slot[t];
+    if (t + 1 < n_tokens && tok_slot[t + 1] == slot) return;      // not its sequence's last row
+    const float* xr = x + (int64_t)t * d;
+    float* s = state + (int64_t)slot * d;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) s[i] = xr[i];
+}
+
+extern "C" int li_token_shift(const float* x, const float* mu, float* state, const int* pos, const int* tok_slot,
+                              void* out, int out_dt, int n_tokens, int d, hipStream_t stream) {
+    if (n_tokens <= 0) return LI_OK;
+    if (d <= 0) return LI_BAD_ARG;
+    dim3 grid(n_tokens), block(d >= 1024 ? 256 : 64);
+    if (out_dt == DT_F32) token_shift_kernel<float><<<grid, block, 0, stream>>>(x, mu, state, pos, tok_slot, (float*)out, d);
+    else if (out_dt == DT_F16) token_shift_kernel<f16><<<grid, block, 0, stream>>>(x, mu, state, pos, tok_slot, (f16*)out, d);
+    else if (out_dt == DT_BF16) token_shift_kernel<bf16><<<grid, block, 0, stream>>>(x, mu, state, pos, tok_slot, (bf16*)out, d);
+    else return LI_BAD_ARG;
+    LI_CHECK_LAUNCH();
+    token_shift_save_kernel<<<grid, block, 0, stream>>>(x, state, tok_slot, d, n_tokens);
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// q, k, v of a step's tokens on their way to an attention over the paged cache.
+//   qkv [T, row_stride] float32: H query heads of d, then G key heads of d, then G value heads of dv
+// q and k: among the first `rot` dimensions of a head, dimension i is paired with i + rot/2 (half layout)
+// or 2j with 2j+1 (adjacent), and the pair (u, v) becomes (u cos a - v sin a, v cos a + u sin a) with
+// a = position * inv_freq[pair]; then, if unit_eps >= 0, the head is divided by sqrt(mean square + unit_eps).
+// q goes to q_out [T, H, dq] (dq >= d, zeros beyond d), k and v into the token's page in the layout of
+// common.h with head sizes dk (>= d, a multiple of 16) and dvp (>= dv, a multiple of 16); what lies beyond
+// d and dv is written as zeros, up to the size the page holds.
+// One wave a head; a lane keeps up to 4 dimensions (heads of up to 256).
+// ---------------------------------------------------------------------------
+template <class T>
+__global__ __launch_bounds__(256) void rope_norm_store_kernel(
+    const float* __restrict__ qkv, int row_stride, const float* __restrict__ inv_freq, int rot, int half_pairing,
+    float unit_eps, const int* __restrict__ pos, const int* __restrict__ tok_slot, Pages c, T* __restrict__ q_out,
+    int H, int G, int d, int dv, int dq, int dk, int dvp) {
+    const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
+    const int p = pos[t];
+    const float* row = qkv + (int64_t)t * row_stride;
+    int64_t page = 0;
+    if (G > 0) page = c.page_table[(int64_t)tok_slot[t] * c.max_pages + p / PAGE];
+    const int tp = p % PAGE, half = rot >> 1;
+    for (int head = wave; head < H + 2 * G; head += n_waves) {
+        if (head < H + G) {
+            const float* src = row + (int64_t)head * d;
+            float val[4];
+            float ss = 0.f;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int i = lane + 64 * u;
+                float v = 0.f;
+                if (i < d) {
+                    v = src[i];
+                    if (i < rot) {
+                        int pair, other;
+                        bool low;
+                        if (half_pairing) { low = i < half; pair = low ? i : i - half; other = low ? i + half : i - half; }
+                        else { low = !(i & 1); pair = i >> 1; other = i ^ 1; }
+                        float sn, cs;
+                        sincosf((float)p * inv_freq[pair], &sn, &cs);
+                        const float o = src[other];
+                        v = low ? v * cs - o * sn : v * cs + o * sn;
+                    }
+                    ss += v * v;
+                }
+                val[u] = v;
+            }
+            if (unit_eps >= 0.f) {
+                const float rms = sqrtf(wave_sum(ss) / (float)d + unit_eps);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) val[u] = val[u] / rms;
+            }
+            if (head < H) {
+                T* q = q_out + ((int64_t)t * H + head) * dq;
+#pragma unroll
+                for (int u = 0; u < 4; ++u) { const int i = lane + 64 * u; if (i < dq) q[i] = from_f32<T>(val[u]); }
+            } else {
+                T* kp = (T*)c.k + page * c.page_stride + (int64_t)(head - H) * k_head_elems(dk);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) { const int i = lane + 64 * u; if (i < dk) kp[k_offset(tp, i, dk)] = from_f32<T>(val[u]); }
+            }
+        } else {
+            const int g = head - H - G;
+            const float* src = row + (int64_t)(H + G) * d + (int64_t)g * dv;
+            T* vp = (T*)c.v + page * c.page_stride + (int64_t)g * v_head_elems(dvp);
+            const int full = round_up(dvp, 32);
+            for (int i = lane; i < full; i += 64) vp[v_offset(tp, i, dvp)] = from_f32<T>(i < dv ? src[i] : 0.f);
+        }
+    }
+}
+
+extern "C" int li_rope_norm_store(const float* qkv, int row_stride, const float* inv_freq, int rot, int half_pairing,
+                                  float unit_eps, const int* pos, const int* tok_slot, const void* k_pages,
+                                  const void* v_pages, int64_t page_stride, const int* page_table, int max_pages,
+                                  void* q_out, int dt, int n_tokens, int H, int G, int d, int dv, int dq, int dk,
+                                  int dvp, hipStream_t stream) {
+    if (n_tokens <= 0) return LI_OK;
+    if (H <= 0 || G < 0 || d <= 0 || d > 256 || dq < d || dq > 256 || rot < 0 || rot > d || (rot & 1)) return LI_BAD_ARG;
+    if (G > 0 && (dv <= 0 || dk < d || dk > 256 || dk % 16 || dvp < dv || dvp % 16 || !page_table)) return LI_BAD_ARG;
+    if (row_stride < (H + G) * d + G * dv || (rot > 0 && !inv_freq)) return LI_BAD_ARG;
+    Pages c{k_pages, v_pages, page_stride, page_table, max_pages};
+    dim3 grid(n_tokens), block(256);
+#define GO(T) rope_norm_store_kernel<T><<<grid, block, 0, stream>>>(qkv, row_stride, inv_freq, rot, half_pairing, \
+        unit_eps, pos, tok_slot, c, (T*)q_out, H, G, d, dv, dq, dk, dvp)
+    if (dt == DT_F32) GO(float); else if (dt == DT_F16) GO(f16); else if (dt == DT_BF16) GO(bf16); else return LI_BAD_ARG;
+#undef GO
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Sigmoid attention, one workgroup per (token, query head), keys in ascending order:
+//   out[t, h, :] = sum over visible j of sigmoid(q_t . k_j * scale + bias[h]) v_j
+// (the weights are not normalised over the keys).  q [T, H, dk] and the cache in the type T, scores,
+// weights and sums in float32; out [T, H, dv] in the type TO.  This is the float32 path's kernel, and the
+// plain form of the 16-bit kernels below.
+// ---------------------------------------------------------------------------
+template <class T, class TO>
+__global__ __launch_bounds__(256) void sigmoid_attn_kernel(
+    const T* __restrict__ q, TO* __restrict__ out, Pages c, const int* __restrict__ pos_of,
+    const int* __restrict__ tok_slot, const float* __restrict__ bias, int H, int G, int dk, int dv, int dvp,
+    float scale, int window) {
+    extern __shared__ float lds[];
+    float* sq = lds;                 // [dk]
+    float* sp = lds + dk;            // [256]
+    const int tid = threadIdx.x;
+    const int64_t tok = blockIdx.x;
+    const int h = blockIdx.y, g = h / (H / G);
+    const int pos = pos_of[tok];
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int* table = c.page_table + (int64_t)tok_slot[tok] * c.max_pages;
+    for (int i = tid; i < dk; i += 256) sq[i] = to_f32(q[(tok * H + h) * dk + i]);
+    __syncthreads();
+    const float b = bias ? bias[h] : 0.f;
+    float acc = 0.f;                 // thread i < dv owns output dimension i
+    for (int t0 = lo; t0 <= pos; t0 += 256) {
+        const int t = t0 + tid;
+        float w = 0.f;
+        if (t <= pos) {
+            const T* kp = (const T*)c.k + (int64_t)table[t / PAGE] * c.page_stride + (int64_t)g * k_head_elems(dk);
+            float dot = 0.f;
+            for (int i = 0; i < dk; ++i) dot = fmaf(sq[i], to_f32(kp[k_offset(t % PAGE, i, dk)]), dot);
+            w = sigmoidf(dot * scale + b);
+        }
+        __syncthreads();
+        sp[tid] = w;
+        __syncthreads();
+        const int n = min(256, pos - t0 + 1);
+        if (tid < dv) {
+            for (int i = 0; i < n; ++i) {
+                const int tt = t0 + i;
+                const T* vp = (const T*)c.v + (int64_t)table[tt / PAGE] * c.page_stride + (int64_t)g * v_head_elems(dvp);
+                acc = fmaf(sp[i], to_f32(vp[v_offset(tt % PAGE, tid, dvp)]), acc);
+            }
+        }
+    }
+    if (tid < dv) out[(tok * H + h) * dv + tid] = from_f32<TO>(acc);
+}
+
+extern "C" int li_sigmoid_attn(const void* q, void* out, int dt, const void* k_pages, const void* v_pages,
+                               int64_t page_stride, const int* page_table, int max_pages, const int* pos,
+                               const int* tok_slot, const float* bias, int n_tokens, int H, int G, int dk, int dv,
+                               int dvp, float scale, int window, hipStream_t stream) {
+    if (n_tokens <= 0) return LI_OK;
+    if (H <= 0 || G <= 0 || H % G || dk <= 0 || dk > 256 || dk % 16 || dv <= 0 || dv > 256 || dvp < dv || dvp % 16)
+        return LI_BAD_ARG;
+    Pages c{k_pages, v_pages, page_stride, page_table, max_pages};
+    dim3 grid(n_tokens, H), block(256);
+    const size_t lds = (size_t)(dk + 256) * sizeof(float);
+#define GO(T) sigmoid_attn_kernel<T, T><<<grid, block, lds, stream>>>((const T*)q, (T*)out, c, pos, tok_slot, bias, \
+        H, G, dk, dv, dvp, scale, window)
+    if (dt == DT_F32) GO(float); else if (dt == DT_F16) GO(f16); else if (dt == DT_BF16) GO(bf16); else return LI_BAD_ARG;
+#undef GO
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Linear attention with a constant decay per head, token by token:
+//   S <- decay[h] * S + k_t v_t^T,   o_t = S^T q_t,        q, k, v = silu of the projections
+// One workgroup per (sequence, head).  The state S [d, dv] of the pair is float32; it is read from
+// `state[slot, h]` when the workgroup starts and written back when the sequence's tokens of this step are
+// done, so a prompt in one step, in portions, or token by token does the same arithmetic in the same order.
+// Thread (rg, j) keeps rows rg*ROWS .. rg*ROWS+ROWS-1 of column j in registers; the partial sums of o over the
+// row groups are added in ascending order through LDS.
+//   proj [T, stride] float32, q at q_off (H heads of d), k at k_off, v at v_off (H heads of dv)
+//   seq_qstart / seq_qlen null: one token per sequence, row i of the step belongs to sequence i (decoding)
+// ---------------------------------------------------------------------------
+template <int ROWS>
+__global__ void decay_attn_kernel(const float* __restrict__ proj, int stride, int q_off, int k_off, int v_off,
+                                  float* __restrict__ state, const float* __restrict__ decay,
+                                  const int* __restrict__ seq_slot, const int* __restrict__ seq_qstart,
+                                  const int* __restrict__ seq_qlen, float* __restrict__ out, int H, int d, int dv) {
+    extern __shared__ float lds[];
+    const int RG = blockDim.x / dv;
+    float* sq = lds;                    // [d]
+    float* sk = sq + d;                 // [d]
+    float* sv = sk + d;                 // [dv]
+    float* red = sv + dv;               // [RG, dv]
+    const int seq = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+    const int j = tid % dv, rg = tid / dv, r0 = rg * ROWS;
+    const int q0 = seq_qstart ? seq_qstart[seq] : seq, n = seq_qlen ? seq_qlen[seq] : 1;
+    float* S = state + (((int64_t)seq_slot[seq] * H + h) * d) * dv;
+    const float lam = decay[h];
+    float s[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) s[r] = r0 + r < d ? S[(int64_t)(r0 + r) * dv + j] : 0.f;
+    for (int t = 0; t < n; ++t) {
+        const float* row = proj + (int64_t)(q0 + t) * stride;
+        __syncthreads();
+        for (int i = tid; i < d; i += blockDim.x) {
+            sq[i] = siluf(row[q_off + h * d + i]);
+            sk[i] = siluf(row[k_off + h * d + i]);
+        }
+        for (int i = tid; i < dv; i += blockDim.x) sv[i] = siluf(row[v_off + h * dv + i]);
+        __syncthreads();
+        const float vj = sv[j];
+        float part = 0.f;
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) {
+            if (r0 + r < d) {
+                s[r] = lam * s[r] + sk[r0 + r] * vj;
+                part += s[r] * sq[r0 + r];
+            }
+        }
+        red[rg * dv + j] = part;
+        __syncthreads();
+        if (rg == 0) {
+            float o = 0.f;
+            for (int g = 0; g < RG; ++g) o += red[g * dv + j];
+            out[(int64_t)(q0 + t) * H * dv + h * dv + j] = o;
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) if (r0 + r < d) S[(int64_t)(r0 + r) * dv + j] = s[r];
+}
+
+extern "C" int li_decay_attn(const float* proj, int stride, int q_off, int k_off, int v_off, float* state,
+                             const float* decay, const int* seq_slot, const int* seq_qstart, const int* seq_qlen,
+                             float* out, int n_seqs, int H, int d, int dv, hipStream_t stream) {
+    if (n_seqs <= 0) return LI_OK;
+    if (H <= 0 || d <= 0 || dv <= 0 || dv > 256 || d > 256) return LI_BAD_ARG;
+    int rows = 4;
+    while (rows < 64 && ((d + rows - 1) / rows) * dv > 512) rows *= 2;
+    const int RG = (d + rows - 1) / rows;
+    if (RG * dv > 1024) return LI_UNSUPPORTED;
+    dim3 grid(n_seqs, H), block(RG * dv);
+    const size_t lds = (size_t)(2 * d + dv + RG * dv) * sizeof(float);
+#define GO(R) decay_attn_kernel<R><<<grid, block, lds, stream>>>(proj, stride, q_off, k_off, v_off, state, decay, \
+        seq_slot, seq_qstart, seq_qlen, out, H, d, dv)
+    if (rows == 4) GO(4); else if (rows == 8) GO(8); else if (rows == 16) GO(16); else if (rows == 32) GO(32); else GO(64);
+#undef GO
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// out = o / sqrt(mean(o^2) + eps) * w * sigmoid(gate): the RMS norm over all heads of a token together, and
+// the gate.  o [T, n] float32; gate: float32 rows of `gate_stride` elements.
+// ---------------------------------------------------------------------------
+template <class TO>
+__global__ void gated_rmsnorm_kernel(const float* __restrict__ o, const float* __restrict__ w,
+                                     const float* __restrict__ gate, int gate_stride, TO* __restrict__ out, int n,
+                                     float eps) {
+    __shared__ float scratch[16];
+    const int64_t t = blockIdx.x;
+    const float* orow = o + t * n;
+    const float* grow = gate + t * gate_stride;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) { const float v = orow[i]; ss += v * v; }
+    const float rms = sqrtf(block_sum(ss, scratch) / (float)n + eps);
+    for (int i = threadIdx.x; i < n; i += blockDim.x)
+        out[t * n + i] = from_f32<TO>(orow[i] / rms * w[i] * sigmoidf(grow[i]));
+}
+
+extern "C" int li_gated_rmsnorm(const float* o, const float* w, const float* gate, int gate_stride, void* out,
+                                int out_dt, int n_rows, int n, float eps, hipStream_t stream) {
+    if (n_rows <= 0) return LI_OK;
+    if (n <= 0 || gate_stride < n) return LI_BAD_ARG;
+    dim3 grid(n_rows), block(n >= 1024 ? 256 : 64);
+    if (out_dt == DT_F32) gated_rmsnorm_kernel<float><<<grid, block, 0, stream>>>(o, w, gate, gate_stride, (float*)out, n, eps);
+    else if (out_dt == DT_F16) gated_rmsnorm_kernel<f16><<<grid, block, 0, stream>>>(o, w, gate, gate_stride, (f16*)out, n, eps);
+    else if (out_dt == DT_BF16) gated_rmsnorm_kernel<bf16><<<grid, block, 0, stream>>>(o, w, gate, gate_stride, (bf16*)out, n, eps);
+    else return LI_BAD_ARG;
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// PolyNorm: out = a N(z) + b N(z^2) + c N(z^3) + e with powers element by element and N the division of a
+// row by its root mean square, sqrt(mean square + eps); coef = (a, b, c, e).  z [T, n] float32.
+// ---------------------------------------------------------------------------
+template <class TO>
+__global__ void polynorm_kernel(const float* __restrict__ z, const float* __restrict__ coef, TO* __restrict__ out,
+                                int n, float eps) {
+    __shared__ float scratch[16];
+    const int64_t t = blockIdx.x;
+    const float* zr = z + t * n;
+    float s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        const float v = zr[i], v2 = v * v, v3 = v2 * v;
+        s1 += v2; s2 += v2 * v2; s3 += v3 * v3;
+    }
+    const float r1 = sqrtf(block_sum(s1, scratch) / (float)n + eps);
+    const float r2 = sqrtf(block_sum(s2, scratch) / (float)n + eps);
+    const float r3 = sqrtf(block_sum(s3, scratch) / (float)n + eps);
+    const float a = coef[0], b = coef[1], c = coef[2], e = coef[3];
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        const float v = zr[i], v2 = v * v, v3 = v2 * v;
+        out[t * n + i] = from_f32<TO>(a * (v / r1) + b * (v2 / r2) + c * (v3 / r3) + e);
+    }
+}
+
+extern "C" int li_polynorm(const float* z, const float* coef, void* out, int out_dt, int n_rows, int n, float eps,
+                           hipStream_t stream) {
+    if (n_rows <= 0) return LI_OK;
+    if (n <= 0) return LI_BAD_ARG;
+    dim3 grid(n_rows), block(n >= 2048 ? 512 : (n >= 256 ? 256 : 64));
+    if (out_dt == DT_F32) polynorm_kernel<float><<<grid, block, 0, stream>>>(z, coef, (float*)out, n, eps);
+    else if (out_dt == DT_F16) polynorm_kernel<f16><<<grid, block, 0, stream>>>(z, coef, (f16*)out, n, eps);
+    else if (out_dt == DT_BF16) polynorm_kernel<bf16><<<grid, block, 0, stream>>>(z, coef, (bf16*)out, n, eps);
+    else return LI_BAD_ARG;
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}

@@ -47,7 +47,8 @@ class Engine:
     def __init__(self, config, model: DecoderModel, max_tokens: int, n_slots: int | None = None, kv_round=None):
         self.config, self.model = config, model
         self.dtype, self.device = model.dtype, model.device
-        self.max_positions = model.spec.max_positions
+        # a design that sets no bound on positions gets the one its cache sets: no sequence outgrows it
+        self.max_positions = model.spec.max_positions or max(1, -(-max_tokens // 64)) * 64
         self.vocab_size = model.spec.vocab_size
         # kv_round="float16" with dtype float32 is the reference's own mix: float32 activations, keys and
         # values rounded to float16 on their way into the cache (src/model/block.cpp:145-148)

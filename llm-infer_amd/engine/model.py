@@ -7,7 +7,7 @@ import torch
 
 from .. import parts as _parts  # noqa: F401  (registers the built-in parts)
 from ..config.spec import ModelSpec
-from ..parts.base import Part, collect_params
+from ..parts.base import Part, cache_specs_of, collect_params
 from ..parts.block import SubLayer
 from ..registry import lookup
 
@@ -38,21 +38,24 @@ class DecoderModel(Part):
                 subs.append(SubLayer(sub.role, part,
                                      None if sub.norm is None else _make("norm", sub.norm, dtype, dev),
                                      None if sub.post_norm is None else _make("norm", sub.post_norm, dtype, dev)))
-            self.layers.append(lookup("block", ls.block)(subs))
+            self.layers.append(lookup("block", ls.block)(subs, **ls.block_params))
             self.layer_mixers.append(mixers)
         self.final_norm = _make("norm", spec.final_norm, dtype, dev)
         self.head = _make("head", spec.head, dtype, dev)
         self.schedule = list(spec.schedule)
-        # what the cache keeps is counted in units: one for each mixer of each run of a layer
+        # what the cache keeps is counted in units: one for each thing that each mixer of each run of a layer
+        # asks of it (one for most mixers; a mixer made of several, or one with a state beside its keys and
+        # values, asks for several: ``cache_specs``)
         self._unit, n = {}, 0
+        self._asks = [[len(cache_specs_of(m)) for m in mixers] for mixers in self.layer_mixers]
+        self._multi = [[hasattr(m, "cache_specs") for m in mixers] for mixers in self.layer_mixers]
         for i, e in enumerate(self.schedule):
-            if e.cache_from is not None and (len(self.layer_mixers[e.layer]) !=
-                                             len(self.layer_mixers[self.schedule[e.cache_from].layer])):
+            if e.cache_from is not None and self._asks[e.layer] != self._asks[self.schedule[e.cache_from].layer]:
                 raise ValueError(f"schedule entry {i} reads the cache of entry {e.cache_from}, whose layer has "
-                                 "another number of mixers")
-            for k in range(len(self.layer_mixers[e.layer])):
-                self._unit[i, k] = n
-                n += 1
+                                 "other mixers")
+            for k, count in enumerate(self._asks[e.layer]):
+                self._unit[i, k] = list(range(n, n + count))
+                n += count
         self._table = collect_params(self)
 
     def _position(self, spec, dtype, dev):
@@ -106,8 +109,8 @@ class DecoderModel(Part):
     def cache_specs(self) -> list:
         """For each unit (each mixer of each schedule entry, in order) what it asks of the cache
         (None: it reads another's)."""
-        return [None if e.cache_from is not None else m.cache_spec()
-                for e in self.schedule for m in self.layer_mixers[e.layer]]
+        return [None if e.cache_from is not None else spec
+                for e in self.schedule for m in self.layer_mixers[e.layer] for spec in cache_specs_of(m)]
 
     # -- the forward pass of one step ---------------------------------------
     def forward(self, ctx, cache) -> torch.Tensor:
@@ -115,7 +118,9 @@ class DecoderModel(Part):
         x = self.embedding.forward(ctx)
         for i, e in enumerate(self.schedule):
             owner = i if e.cache_from is None else e.cache_from
-            views = [cache.view(self._unit[owner, k]) for k in range(len(self.layer_mixers[e.layer]))]
+            # one view for a mixer, or the list of its views for one that asks several things of the cache
+            views = [[cache.view(u) for u in self._unit[owner, k]] if multi else cache.view(self._unit[owner, k][0])
+                     for k, multi in enumerate(self._multi[e.layer])]
             layer = self.layers[e.layer]
             if getattr(layer, "takes_next_norm", False):
                 # the norm that reads the residual stream after this layer: the next layer's first

@@ -1,6 +1,7 @@
 """Compiles the HIP sources for gfx950 into shared libraries and loads them.
 
-``libli_core.so`` holds every kernel whose sizes are run-time values; the
+``libli_core.so`` holds every kernel of the softmax decoder whose sizes are run-time
+values, ``libli_mixers.so`` those of the other mixers, norms and activations; the
 attention kernels are compiled once per head size (``libli_attn_hd<N>.so``), at
 the first call that needs that size.  Libraries are kept beside the sources (or in
 a temporary folder when that is not writable) with a stamp of the sources they
@@ -24,6 +25,7 @@ CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
 ARCH = "gfx950"
 CORE_SOURCES = ("elementwise.hip", "gemm.hip", "gemm_prefill.hip", "sampling.hip")
 ATTN_SOURCE = "attention.hip"
+MIXER_SOURCES = ("mixers.hip",)
 # the headers a library's sources include (its stamp covers them)
 HEADERS = {"libli_core.so": ("common.h", "gemm_common.h", "no_alloc.h")}
 DEFAULT_HEADERS = ("common.h",)
@@ -183,9 +185,16 @@ def attention_library(head_dim: int, force=False):
     return _load(f"libli_attn_hd{head_dim}.so", (ATTN_SOURCE,), (f"-DHEAD_DIM={head_dim}",), force)
 
 
+def mixers_library(force=False):
+    """The kernels of the other mixers and arrangements (csrc/mixers.hip): a library of its own, so that a
+    model is not kept waiting for kernels that it does not run."""
+    return _load("libli_mixers.so", MIXER_SOURCES, (), force)
+
+
 def build_all(head_dims=(16, 32, 48, 64, 128), force=True) -> None:
-    """Compile the core library and the attention library for each head size given."""
+    """Compile the core library, the mixers' library and the attention library for each head size given."""
     core_library(force=force)
+    mixers_library(force=force)
     with ThreadPoolExecutor(max_workers=4) as pool:
         list(pool.map(lambda hd: _build_library(f"libli_attn_hd{hd}.so", (ATTN_SOURCE,),
                                                 (f"-DHEAD_DIM={hd}",), force), head_dims))

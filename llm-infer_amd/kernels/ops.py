@@ -803,3 +803,193 @@ def gemv_tiled(x, w: Tensor, mode=EPI_STORE, out_dtype=None, nt=0, kw=0):
     _check(core().li_gemv_tiled(_ptr(x), _ptr(w), DT[x.dtype], _ptr(out), DT[out.dtype], mode, m, n, k,
                                 nt, kw, None, None, None, _stream()), "gemv_tiled")
     return out
+
+
+# ---------------------------------------------------------------------------
+# the other mixers, norms and activations (csrc/mixers.hip)
+# ---------------------------------------------------------------------------
+_mixers = None
+
+
+def mixers():
+    global _mixers
+    if _mixers is None:
+        _mixers = build.mixers_library()
+    return _mixers
+
+
+def _f32_rows(x, what):
+    _need(x.dtype == torch.float32 and x.dim() == 2, f"{what}: float32 [T, n]")
+
+
+def layernorm(x: torch.Tensor, w: torch.Tensor, eps: float, out_dtype, rows: torch.Tensor | None = None) -> torch.Tensor:
+    """out[r] = (x[rows[r]] - mean) / sqrt(var + eps) * w, float32 inside; no bias."""
+    _dev(x, w, rows)
+    _f32_rows(x, "layernorm x")
+    _need(w.dtype == torch.float32 and w.shape == (x.shape[1],), "norm weight: float32 [d]")
+    if rows is not None:
+        _need(rows.dtype == torch.int32, "rows: int32")
+    n = x.shape[0] if rows is None else rows.numel()
+    out = torch.empty((n, x.shape[1]), dtype=out_dtype, device=x.device)
+    _check(mixers().li_layernorm(_ptr(x), _ptr(w), _ptr(rows), _ptr(out), DT[out_dtype], n, x.shape[1], c_float(eps),
+                                 _stream()), "layernorm")
+    return out
+
+
+def add_layernorm(x, alpha: float, addends, w, eps: float, copy_dtype=None):
+    """x <- LN(alpha * x + sum of scale_i * y_i) * w in place on the float32 rows of ``x``; ``addends``: one or
+    two (y, scale) with y float32 of x's shape.  ``copy_dtype`` (a 16-bit type): the new rows are returned in
+    that type as well (else None)."""
+    _need(1 <= len(addends) <= 2, "add_layernorm: one or two addends")
+    (y1, s1), (y2, s2) = addends[0], (addends[1] if len(addends) > 1 else (None, 0.0))
+    _dev(x, y1, y2, w)
+    _f32_rows(x, "add_layernorm x")
+    for y in (y1, y2):
+        _need(y is None or (y.dtype == torch.float32 and y.shape == x.shape), "add_layernorm: addends float32 like x")
+    _need(w.dtype == torch.float32 and w.shape == (x.shape[1],), "norm weight: float32 [d]")
+    _drop_row_stats(x)
+    copy = None
+    if copy_dtype is not None and copy_dtype != torch.float32:
+        copy = torch.empty(x.shape, dtype=copy_dtype, device=x.device)
+    _check(mixers().li_add_layernorm(_ptr(x), c_float(alpha), _ptr(y1), c_float(s1), _ptr(y2), c_float(s2), _ptr(w),
+                                     c_float(eps), _ptr(copy), DT[copy.dtype] if copy is not None else 0, x.shape[0],
+                                     x.shape[1], _stream()), "add_layernorm")
+    return copy
+
+
+def add_scaled(x, addends) -> None:
+    """x += sum of scale_i * y_i (one or two addends, float32 of x's shape)."""
+    _need(1 <= len(addends) <= 2, "add_scaled: one or two addends")
+    (y1, s1), (y2, s2) = addends[0], (addends[1] if len(addends) > 1 else (None, 0.0))
+    _dev(x, y1, y2)
+    for y in (x, y1, y2):
+        _need(y is None or (y.dtype == torch.float32 and y.shape == x.shape), "add_scaled: float32 tensors of one shape")
+    _drop_row_stats(x)
+    _check(mixers().li_add_scaled(_ptr(x), _ptr(y1), c_float(s1), _ptr(y2), c_float(s2), c_int64(x.numel()), _stream()),
+           "add_scaled")
+
+
+def cast(x: torch.Tensor, dtype) -> torch.Tensor:
+    """float32 -> a 16-bit type (a float32 ``dtype`` gives ``x`` itself back)."""
+    if dtype == torch.float32:
+        return x
+    _dev(x)
+    _need(x.dtype == torch.float32 and dtype in (torch.float16, torch.bfloat16), "cast: float32 to a 16-bit type")
+    out = torch.empty(x.shape, dtype=dtype, device=x.device)
+    _check(mixers().li_cast(_ptr(x), _ptr(out), DT[dtype], c_int64(x.numel()), _stream()), "cast")
+    return out
+
+
+def token_shift(x, mu, state, pos, tok_slot, out_dtype) -> torch.Tensor:
+    """out_t = x_t + (x_{t-1} - x_t) * mu with the row before from this step or from ``state[slot]`` (zeros at
+    position 0); afterwards ``state[slot]`` holds each sequence's last row of this step."""
+    _dev(x, mu, state, pos, tok_slot)
+    _f32_rows(x, "token_shift x")
+    t, d = x.shape
+    _need(mu.dtype == torch.float32 and mu.shape == (d,), "token_shift: float32 [d] mixing weights")
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] == d, "token_shift: state float32 [slots, d]")
+    _need(pos.dtype == torch.int32 and tok_slot.dtype == torch.int32 and pos.numel() >= t and tok_slot.numel() >= t,
+          "token_shift: int32 positions and slots for every token")
+    out = torch.empty((t, d), dtype=out_dtype, device=x.device)
+    _check(mixers().li_token_shift(_ptr(x), _ptr(mu), _ptr(state), _ptr(pos), _ptr(tok_slot), _ptr(out), DT[out_dtype],
+                                   t, d, _stream()), "token_shift")
+    return out
+
+
+def rope_norm_store(qkv, inv_freq, rotary_dim, half_pairing, unit_eps, pos, tok_slot, kv, n_heads, n_kv_heads,
+                    head_dim, v_head_dim, q_dim, k_dim, v_dim, out_dtype) -> torch.Tensor:
+    """q and k of a step rotated by position (half or adjacent pairing), then, with ``unit_eps`` not None,
+    divided by their root mean square per head; k and v written into the pages (``kv`` = (k_pages, v_pages,
+    page_stride, page_table); head sizes ``k_dim`` and ``v_dim`` in the pages, zeros beyond the true ones).
+    Returns q [T, H, q_dim]."""
+    k_pages, v_pages, page_stride, page_table = kv
+    _dev(qkv, inv_freq, pos, tok_slot, k_pages, v_pages, page_table)
+    _f32_rows(qkv, "rope_norm_store qkv")
+    t = qkv.shape[0]
+    _need(qkv.shape[1] >= (n_heads + n_kv_heads) * head_dim + n_kv_heads * v_head_dim, "qkv row too short")
+    _need(pos.dtype == torch.int32 and tok_slot.dtype == torch.int32 and pos.numel() >= t and tok_slot.numel() >= t,
+          "int32 positions and slots for every token")
+    _need(max(head_dim, q_dim, k_dim, v_dim) <= 256 and q_dim >= head_dim and k_dim >= head_dim and v_dim >= v_head_dim
+          and k_dim % 16 == 0 and v_dim % 16 == 0, "head sizes up to 256, padded sizes multiples of 16")
+    if rotary_dim > 0:
+        _need(inv_freq is not None and inv_freq.dtype == torch.float32 and inv_freq.numel() >= rotary_dim // 2,
+              "inv_freq: float32 [rotary_dim / 2]")
+    _need(k_pages.dtype == out_dtype and v_pages.dtype == out_dtype, "cache dtype differs from q dtype")
+    _need(page_table.dtype == torch.int32 and page_table.dim() == 2, "page_table: int32 [slots, pages]")
+    q = torch.empty((t, n_heads, q_dim), dtype=out_dtype, device=qkv.device)
+    _check(mixers().li_rope_norm_store(
+        _ptr(qkv), qkv.shape[1], _ptr(inv_freq), rotary_dim, int(half_pairing),
+        c_float(-1.0 if unit_eps is None else unit_eps), _ptr(pos), _ptr(tok_slot), _ptr(k_pages), _ptr(v_pages),
+        c_int64(page_stride), _ptr(page_table), page_table.shape[1], _ptr(q), DT[out_dtype], t, n_heads, n_kv_heads,
+        head_dim, v_head_dim, q_dim, k_dim, v_dim, _stream()), "rope_norm_store")
+    return q
+
+
+def sigmoid_attention(q, kv, pos, tok_slot, bias, n_heads, n_kv_heads, k_dim, v_head_dim, v_dim, scale, window=None):
+    """out[t, h] = sum over visible keys j of sigmoid(q_t . k_j * scale + bias[h]) v_j (no normalisation over
+    the keys); q [T, H, k_dim] and the pages in one type, scores and weights float32.  Returns [T, H, v_head_dim]."""
+    k_pages, v_pages, page_stride, page_table = kv
+    _dev(q, k_pages, v_pages, page_table, pos, tok_slot, bias)
+    _need(q.dtype in DT and q.dim() == 3 and q.shape[1:] == (n_heads, k_dim), "q: [T, H, k_dim]")
+    _check_pages(k_pages, v_pages, page_table, n_kv_heads, k_dim, q.dtype)
+    _need(n_heads % n_kv_heads == 0, "query heads: a multiple of the key/value heads")
+    _need(pos.numel() >= q.shape[0] and tok_slot.numel() >= q.shape[0], "per-token arrays too short")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == n_heads), "bias: float32 [H]")
+    out = torch.empty((q.shape[0], n_heads, v_head_dim), dtype=q.dtype, device=q.device)
+    _check(mixers().li_sigmoid_attn(_ptr(q), _ptr(out), DT[q.dtype], _ptr(k_pages), _ptr(v_pages), c_int64(page_stride),
+                                    _ptr(page_table), page_table.shape[1], _ptr(pos), _ptr(tok_slot), _ptr(bias),
+                                    q.shape[0], n_heads, n_kv_heads, k_dim, v_head_dim, v_dim, c_float(scale),
+                                    int(window or 0), _stream()), "sigmoid_attn")
+    return out
+
+
+def decay_attention(proj, q_off, k_off, v_off, state, decay, seq_slot, seq_qstart, seq_qlen, n_seqs, n_heads,
+                    head_dim, v_head_dim) -> torch.Tensor:
+    """Linear attention with a constant decay per head over the tokens of a step, from and into the float32
+    ``state`` [slots, H, d, dv]: S <- decay S + k v^T, o = S^T q, with q, k, v = silu of the columns of ``proj``
+    (float32 [T, n]) at the given offsets.  ``seq_qstart`` / ``seq_qlen`` None: one token per sequence.
+    Returns float32 [T, H * dv]."""
+    _dev(proj, state, decay, seq_slot, seq_qstart, seq_qlen)
+    _f32_rows(proj, "decay_attention proj")
+    H, d, dv = n_heads, head_dim, v_head_dim
+    _need(state.dtype == torch.float32 and tuple(state.shape[1:]) == (H, d, dv), "state: float32 [slots, H, d, dv]")
+    _need(decay.dtype == torch.float32 and decay.numel() == H, "decay: float32 [H]")
+    _need(max(q_off + H * d, k_off + H * d, v_off + H * dv) <= proj.shape[1], "decay_attention: columns outside proj")
+    _need(seq_slot.dtype == torch.int32 and seq_slot.numel() >= n_seqs, "seq_slot: int32 [sequences]")
+    if seq_qstart is None:
+        _need(seq_qlen is None and proj.shape[0] >= n_seqs, "one token per sequence needs a row for each")
+    else:
+        _need(seq_qlen is not None and seq_qstart.dtype == torch.int32 and seq_qlen.dtype == torch.int32 and
+              seq_qstart.numel() >= n_seqs and seq_qlen.numel() >= n_seqs, "seq_qstart, seq_qlen: int32 [sequences]")
+    out = torch.empty((proj.shape[0], H * dv), dtype=torch.float32, device=proj.device)
+    _check(mixers().li_decay_attn(_ptr(proj), proj.shape[1], q_off, k_off, v_off, _ptr(state), _ptr(decay),
+                                  _ptr(seq_slot), _ptr(seq_qstart), _ptr(seq_qlen), _ptr(out), n_seqs, H, d, dv,
+                                  _stream()), "decay_attn")
+    return out
+
+
+def gated_rmsnorm(o, w, gate_rows, gate_off, eps, out_dtype) -> torch.Tensor:
+    """o / sqrt(mean(o^2) + eps) * w * sigmoid(gate): o float32 [T, n]; the gate is columns gate_off .. gate_off + n
+    of the float32 rows ``gate_rows``."""
+    _dev(o, w, gate_rows)
+    _f32_rows(o, "gated_rmsnorm o")
+    _f32_rows(gate_rows, "gated_rmsnorm gate")
+    t, n = o.shape
+    _need(w.dtype == torch.float32 and w.shape == (n,), "norm weight: float32 [n]")
+    _need(gate_rows.shape[0] == t and gate_off + n <= gate_rows.shape[1], "gate columns outside their rows")
+    out = torch.empty((t, n), dtype=out_dtype, device=o.device)
+    gate = gate_rows.view(-1)[gate_off:]
+    _check(mixers().li_gated_rmsnorm(_ptr(o), _ptr(w), _ptr(gate), gate_rows.shape[1], _ptr(out), DT[out_dtype], t, n,
+                                     c_float(eps), _stream()), "gated_rmsnorm")
+    return out
+
+
+def polynorm(z, coef, eps, out_dtype) -> torch.Tensor:
+    """a N(z) + b N(z^2) + c N(z^3) + e over float32 rows; coef float32 [4] = (a, b, c, e)."""
+    _dev(z, coef)
+    _f32_rows(z, "polynorm z")
+    _need(coef.dtype == torch.float32 and coef.numel() == 4, "polynorm: float32 [4] coefficients")
+    out = torch.empty(z.shape, dtype=out_dtype, device=z.device)
+    _check(mixers().li_polynorm(_ptr(z), _ptr(coef), _ptr(out), DT[out_dtype], z.shape[0], z.shape[1], c_float(eps),
+                                _stream()), "polynorm")
+    return out

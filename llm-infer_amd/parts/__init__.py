@@ -1,10 +1,15 @@
 from .base import Part, collect_params
-from .norm import RMSNorm
+from .norm import LayerNorm, RMSNorm
 from .position import RotaryPosition, NoPosition
 from .attention import Attention
-from .feed_forward import GatedMLP
+from .feed_forward import GatedMLP, PolyNormMLP
+from .token_shift import ShiftedMixer
+from .parallel import ParallelMixers
+from .sigmoid_attention import SigmoidAttention
+from .decay_attention import DecayLinearAttention
 from .embedding import Embedding, LMHead
-from .block import Block, PreNormBlock, SubLayer
+from .block import Block, PostNormBlock, PreNormBlock, SubLayer
 
 __all__ = ["Part", "collect_params", "RMSNorm", "RotaryPosition", "NoPosition", "Attention", "GatedMLP",
-           "Embedding", "LMHead", "Block", "PreNormBlock", "SubLayer"]
+           "Embedding", "LMHead", "Block", "PreNormBlock", "SubLayer", "LayerNorm", "PolyNormMLP", "ShiftedMixer",
+           "ParallelMixers", "SigmoidAttention", "DecayLinearAttention", "PostNormBlock"]

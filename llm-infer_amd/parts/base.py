@@ -31,6 +31,21 @@ class Part:
         return []
 
 
+def cache_specs_of(mixer) -> list:
+    """What a mixer asks of the cache, as a list: ``cache_specs()`` of a mixer that asks for several things (it
+    is then handed the list of its views, in that order), else the one ``cache_spec()``."""
+    if hasattr(mixer, "cache_specs"):
+        return list(mixer.cache_specs())
+    return [mixer.cache_spec()]
+
+
+def views_for(mixer, views: list, at: int = 0):
+    """From the flat list ``views`` of a composite mixer, what its child ``mixer`` is handed (its specs begin at
+    index ``at``), and the index behind them."""
+    n = len(cache_specs_of(mixer))
+    return (views[at:at + n] if hasattr(mixer, "cache_specs") else views[at]), at + n
+
+
 def collect_params(part: Part, out: dict | None = None) -> dict:
     """Full tensor name -> (owning part, local name, ParamSpec) for a part and all below it."""
     out = {} if out is None else out

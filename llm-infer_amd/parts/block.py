@@ -1,5 +1,7 @@
 from __future__ import annotations
 
+import torch
+
 from ..kernels import ops
 from ..registry import register_block
 from .base import Part
@@ -89,3 +91,54 @@ class PreNormBlock(Block):
                 s.part.forward(h, ctx, next(views), x, owns_cache)
             else:
                 s.part.forward(h, x)
+
+
+@register_block("post_norm")
+class PostNormBlock(Block):
+    """x <- norm(alpha * x + part(x)) for each sub-layer in turn: the parts read the residual stream itself and
+    the norm comes after the sum; ``alpha`` scales the stream's own share.  Every sub-layer has a norm on its
+    output (a layer norm with a weight, ``parts.norm.LayerNorm``) and none on its input.
+
+    A part may hand over what it adds as ``addends(h, ...) -> [(y, scale), ...]`` (float32 rows of the
+    stream's shape); the scaled sum, the stream's share and the norm are then one kernel.  A part without
+    ``addends`` adds into a cleared buffer through its ``forward``.  A part that says ``reads_residual`` takes
+    the float32 rows as they are; the others get them in the compute dtype, a copy that the norm kernel of
+    the sub-layer before writes along."""
+
+    def __init__(self, sublayers, alpha: float = 1.0):
+        super().__init__(sublayers)
+        self.alpha = float(alpha)
+        for s in self.sublayers:
+            if s.norm is not None or s.post_norm is None or not hasattr(s.post_norm, "weight"):
+                raise ValueError("a post_norm block has one norm with a weight after each part and none before it")
+
+    @staticmethod
+    def _addends(s, h, x, ctx, view, owns_cache):
+        if hasattr(s.part, "addends"):
+            return s.part.addends(h, ctx, view, owns_cache) if s.role == "mixer" else s.part.addends(h)
+        y = torch.zeros_like(x)
+        if s.role == "mixer":
+            s.part.forward(h, ctx, view, y, owns_cache)
+        else:
+            s.part.forward(h, y)
+        return [(y, 1.0)]
+
+    def forward(self, x, ctx, cache_views, owns_cache=True):
+        views = iter(cache_views)
+        copy = None                                  # the rows of x in the compute dtype, if the last norm left them
+        for i, s in enumerate(self.sublayers):
+            dtype = s.post_norm.dtype
+            if getattr(s.part, "reads_residual", False):
+                h = x
+            else:
+                h = copy if copy is not None and copy.dtype == dtype else ops.cast(x, dtype)
+            adds = self._addends(s, h, x, ctx, next(views) if s.role == "mixer" else None, owns_cache)
+            while len(adds) > 2:                     # the norm kernel takes two: sum the rest beforehand
+                (y0, s0), rest = adds[0], adds[1:3]
+                y0 = y0 * s0 if s0 != 1.0 else y0
+                ops.add_scaled(y0, rest)
+                adds = [(y0, 1.0)] + adds[3:]
+            nxt = self.sublayers[i + 1] if i + 1 < len(self.sublayers) else None
+            wants_copy = nxt is not None and not getattr(nxt.part, "reads_residual", False)
+            copy = ops.add_layernorm(x, self.alpha, adds, s.post_norm.weight, s.post_norm.eps,
+                                     nxt.post_norm.dtype if wants_copy else None)

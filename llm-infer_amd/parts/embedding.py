@@ -12,16 +12,16 @@ from .base import Part
 class Embedding(Part):
     """x = float32(table[token]), unscaled (src/model/model.cpp:101-118)."""
 
-    def __init__(self, *, vocab_size, hidden_size, prefix, dtype, device):
-        self.vocab_size, self.hidden_size = vocab_size, hidden_size
+    def __init__(self, *, vocab_size, hidden_size, name="weight", prefix, dtype, device):
+        self.vocab_size, self.hidden_size, self.name = vocab_size, hidden_size, name
         self.prefix, self.dtype, self.device = prefix, dtype, device
         self.weight = None
 
     def params(self):
-        return {"weight": ParamSpec((self.vocab_size, self.hidden_size))}
+        return {self.name: ParamSpec((self.vocab_size, self.hidden_size))}
 
     def bind(self, tensors):
-        self.weight = tensors["weight"]
+        self.weight = tensors[self.name]
 
     def forward(self, ctx):
         """The residual stream's first value for the step's tokens, float32 [T, hidden].  ``ctx`` is the

@@ -45,3 +45,34 @@ class GatedMLP(Part):
     def forward(self, h, residual):
         t = ops.linear(h, self.w_gate_up, self.mode, out_dtype=self.dtype)
         ops.linear(t, self.w_down, ops.EPI_ADD, out=residual)
+
+
+@register_feed_forward("poly_mlp")
+class PolyNormMLP(Part):
+    """down(PolyNorm(up(x))): no gate.  PolyNorm(z) = a N(z) + b N(z^2) + c N(z^3) + e with the powers taken
+    element by element and N the division of a token's vector by its root mean square (``eps`` inside the
+    root), computed in float32; (a, b, c, e) are the four numbers of the tensor ``names["act"]``."""
+
+    def __init__(self, *, hidden_size, intermediate_size, eps, names=None, prefix, dtype, device):
+        self.hidden_size, self.intermediate_size, self.eps = hidden_size, intermediate_size, float(eps)
+        self.names = {"up": "up_proj.weight", "down": "down_proj.weight", "act": "act", **(names or {})}
+        self.prefix, self.dtype, self.device = prefix, dtype, device
+        self.w_up = self.w_down = self.coef = None
+
+    def params(self):
+        f, d, n = self.intermediate_size, self.hidden_size, self.names
+        return {n["up"]: ParamSpec((f, d)), n["down"]: ParamSpec((d, f)), n["act"]: ParamSpec((4,), "vector", "ones")}
+
+    def bind(self, tensors):
+        n = self.names
+        self.w_up, self.w_down = ops.prepare_weight(tensors[n["up"]]), ops.prepare_weight(tensors[n["down"]])
+        self.coef = tensors[n["act"]]
+
+    def addends(self, h):
+        z = ops.linear(h, self.w_up, out_dtype=torch.float32)
+        a = ops.polynorm(z, self.coef, self.eps, self.dtype)
+        return [(ops.linear(a, self.w_down, out_dtype=torch.float32), 1.0)]
+
+    def forward(self, h, residual):
+        ops.linear(ops.polynorm(ops.linear(h, self.w_up, out_dtype=torch.float32), self.coef, self.eps, self.dtype),
+                   self.w_down, ops.EPI_ADD, out=residual)

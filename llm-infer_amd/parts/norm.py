@@ -37,3 +37,23 @@ class RMSNorm(Part):
             if ready is not None:
                 return ready
         return ops.rmsnorm(x, self.weight, self.eps, self.dtype, rows)
+
+
+@register_norm("layernorm")
+class LayerNorm(Part):
+    """out = (x - mean) / sqrt(var + eps) * weight in float32, var the mean of the squared deviations; a weight
+    and no bias.  ``name`` is the local name of the weight's tensor."""
+
+    def __init__(self, *, size: int, eps: float, name: str = "weight", prefix: str, dtype, device):
+        self.size, self.eps, self.name = size, float(eps), name
+        self.prefix, self.dtype, self.device = prefix, dtype, device
+        self.weight = None
+
+    def params(self):
+        return {self.name: ParamSpec((self.size,), "vector", "ones")}
+
+    def bind(self, tensors):
+        self.weight = tensors[self.name]
+
+    def forward(self, x: torch.Tensor, rows: torch.Tensor | None = None):
+        return ops.layernorm(x, self.weight, self.eps, self.dtype, rows)

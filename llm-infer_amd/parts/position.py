@@ -13,6 +13,7 @@ class RotaryPosition(Part):
     that starts at dimension i (include/kernels_cpu.hpp:82-100).  ``pairing`` "adjacent"
     rotates (i, i+1) as the reference does; "half" rotates (i/2, i/2 + rotary_dim/2), the order of
     a checkpoint whose q and k rows were never permuted for the reference (docs/gguf.md:487-493).
+    ``scaling_factor`` divides every frequency (linear scaling of positions).
 
     The kernels rotate adjacent pairs only.  A half-paired model runs on them unchanged because a
     score is a sum over the dimensions of a head and does not care about their order: the mixer asks
@@ -29,13 +30,17 @@ class RotaryPosition(Part):
     k and v into the layer's pages, and return q.
     """
 
-    def __init__(self, *, theta: float, rotary_dim: int, head_dim: int, pairing: str = "adjacent", prefix: str = "",
-                 dtype, device):
+    def __init__(self, *, theta: float, rotary_dim: int, head_dim: int, pairing: str = "adjacent",
+                 scaling_factor: float = 1.0, prefix: str = "", dtype, device):
         self.rotary_dim, self.head_dim, self.pairing, self.theta = rotary_dim, head_dim, pairing, float(theta)
+        self.scaling_factor = float(scaling_factor)
         self.prefix = prefix
         i = torch.arange(0, rotary_dim, 2, dtype=torch.float32)
         # 1 / powf(theta, i / rotary_dim) in float32, as kernels_cpu.hpp:87
         inv = 1.0 / torch.pow(torch.tensor(float(theta), dtype=torch.float32), i / float(rotary_dim))
+        if self.scaling_factor != 1.0:
+            # linear scaling: every frequency divided by the factor, i.e. positions counted in its units
+            inv = inv / self.scaling_factor
         self.inv_freq = inv.to(device) if device is not None else inv
         self.dtype = dtype
 

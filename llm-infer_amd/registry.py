@@ -58,8 +58,10 @@ def lookup(table_name: str, kind: str):
 
 def config_from_dict(raw: dict):
     archs = raw.get("architectures")
+    if not archs and isinstance(raw.get("architecture"), str):
+        archs = [raw["architecture"]]             # some designs name theirs under the singular key
     if not archs:
-        raise ConfigError("config.json names no architecture (key 'architectures'); known: "
+        raise ConfigError("config.json names no architecture (key 'architectures' or 'architecture'); known: "
                           + ", ".join(sorted(ARCHITECTURES)))
     name = archs[0]
     if name not in ARCHITECTURES:
