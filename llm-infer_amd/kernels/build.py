@@ -191,10 +191,30 @@ def mixers_library(force=False):
     return _load("libli_mixers.so", MIXER_SOURCES, (), force)
 
 
-def build_all(head_dims=(16, 32, 48, 64, 128), force=True) -> None:
-    """Compile the core library, the mixers' library and the attention library for each head size given."""
+SIGMOID_ATTN_SOURCE = "sigmoid_attention.hip"
+
+
+def _sigmoid_attention_args(key_dim: int, value_dim: int):
+    for n in (key_dim, value_dim):
+        if n % 16 != 0 or not 16 <= n <= 256:
+            raise BuildError(f"head size {n}: the sigmoid attention kernels take multiples of 16 up to 256")
+    return (f"libli_sigattn_k{key_dim}_v{value_dim}.so", (SIGMOID_ATTN_SOURCE,),
+            (f"-DKEY_DIM={key_dim}", f"-DVALUE_DIM={value_dim}"))
+
+
+def sigmoid_attention_library(key_dim: int, value_dim: int, force=False):
+    """The matrix-core kernels of sigmoid attention for one pair of head sizes (keys, values), compiled at the
+    first call that needs the pair."""
+    return _load(*_sigmoid_attention_args(key_dim, value_dim), force)
+
+
+def build_all(head_dims=(16, 32, 48, 64, 128), force=True, sigmoid_head_dims=((48, 32), (128, 128))) -> None:
+    """Compile the core library, the mixers' library, the attention library for each head size given and the
+    sigmoid attention library for each pair of head sizes given."""
     core_library(force=force)
     mixers_library(force=force)
+    for kd, vd in sigmoid_head_dims:
+        _build_library(*_sigmoid_attention_args(kd, vd), force)
     with ThreadPoolExecutor(max_workers=4) as pool:
         list(pool.map(lambda hd: _build_library(f"libli_attn_hd{hd}.so", (ATTN_SOURCE,),
                                                 (f"-DHEAD_DIM={hd}",), force), head_dims))

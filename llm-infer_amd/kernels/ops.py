@@ -943,6 +943,62 @@ def sigmoid_attention(q, kv, pos, tok_slot, bias, n_heads, n_kv_heads, k_dim, v_
     return out
 
 
+_sigattn: dict = {}
+
+
+def _sigattn_lib(key_dim: int, value_dim: int):
+    lib = _sigattn.get((key_dim, value_dim))
+    if lib is None:
+        lib = build.sigmoid_attention_library(key_dim, value_dim)
+        _need(lib.li_sigattn_key_dim() == key_dim and lib.li_sigattn_value_dim() == value_dim,
+              "sigmoid attention library built for other head sizes")
+        _sigattn[key_dim, value_dim] = lib
+    return lib
+
+
+def _sigattn_check(q, kv, bias, n_heads, n_kv_heads, k_dim, v_head_dim, v_dim):
+    k_pages, v_pages, page_stride, page_table = kv
+    _dev(q, k_pages, v_pages, page_table, bias)
+    _need(q.dtype in (torch.float16, torch.bfloat16) and q.dim() == 3 and q.shape[1:] == (n_heads, k_dim),
+          "q: 16-bit [T, H, k_dim]")
+    _check_pages(k_pages, v_pages, page_table, n_kv_heads, k_dim, q.dtype)
+    _need(n_heads % n_kv_heads == 0 and 0 < v_head_dim <= v_dim, "heads and head sizes do not fit")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == n_heads), "bias: float32 [H]")
+    return k_pages, v_pages, page_stride, page_table
+
+
+def sigmoid_attention_prefill(q, kv, meta, bias, n_heads, n_kv_heads, k_dim, v_head_dim, v_dim, scale, window=None):
+    """16-bit sigmoid attention for a step with prompts (or portions of prompts) on the matrix cores; ``meta`` as
+    for ``attention_prefill``.  Returns [T, H, v_head_dim]."""
+    k_pages, v_pages, page_stride, page_table = _sigattn_check(q, kv, bias, n_heads, n_kv_heads, k_dim, v_head_dim, v_dim)
+    out = torch.empty((q.shape[0], n_heads, v_head_dim), dtype=q.dtype, device=q.device)
+    _check(_sigattn_lib(k_dim, v_dim).li_sigattn_prefill(
+        _ptr(q), _ptr(out), DT[q.dtype], _ptr(k_pages), _ptr(v_pages), c_int64(page_stride), _ptr(page_table),
+        page_table.shape[1], _ptr(meta["tile_seq"]), _ptr(meta["tile_q0"]), meta["n_tiles"], _ptr(meta["seq_slot"]),
+        _ptr(meta["seq_qstart"]), _ptr(meta["seq_qlen"]), _ptr(meta["seq_ctx"]), _ptr(bias), n_heads, n_kv_heads,
+        v_head_dim, c_float(scale), int(window or 0), _stream()), "sigattn_prefill")
+    return out
+
+
+def sigmoid_attention_decode(q, kv, seq_slot, seq_ctx, n_seqs, bias, n_heads, n_kv_heads, k_dim, v_head_dim, v_dim,
+                             scale, window=None, splits: int = 1):
+    """16-bit sigmoid attention for one new token per sequence; q [B, H, k_dim].  The context is cut into
+    ``splits`` parts whose sums are added in ascending order."""
+    k_pages, v_pages, page_stride, page_table = _sigattn_check(q, kv, bias, n_heads, n_kv_heads, k_dim, v_head_dim, v_dim)
+    _dev(seq_slot, seq_ctx)
+    _need(q.shape[0] == n_seqs and seq_slot.numel() >= n_seqs and seq_ctx.numel() >= n_seqs, "per-sequence arrays too short")
+    _need(1 <= splits <= 64, f"sigmoid_attention_decode: {splits} splits")
+    out = torch.empty((n_seqs, n_heads, v_head_dim), dtype=q.dtype, device=q.device)
+    part = None
+    if splits > 1:
+        part = torch.empty((n_seqs, n_heads, splits, v_head_dim), dtype=torch.float32, device=q.device)
+    _check(_sigattn_lib(k_dim, v_dim).li_sigattn_decode(
+        _ptr(q), _ptr(out), DT[q.dtype], _ptr(k_pages), _ptr(v_pages), c_int64(page_stride), _ptr(page_table),
+        page_table.shape[1], _ptr(seq_slot), _ptr(seq_ctx), _ptr(bias), n_seqs, n_heads, n_kv_heads, v_head_dim,
+        c_float(scale), int(window or 0), splits, _ptr(part), _stream()), "sigattn_decode")
+    return out
+
+
 def decay_attention(proj, q_off, k_off, v_off, state, decay, seq_slot, seq_qstart, seq_qlen, n_seqs, n_heads,
                     head_dim, v_head_dim) -> torch.Tensor:
     """Linear attention with a constant decay per head over the tokens of a step, from and into the float32

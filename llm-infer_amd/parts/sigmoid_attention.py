@@ -75,8 +75,15 @@ class SigmoidAttention(Part):
         kv = view.as_tuple()
         q = ops.rope_norm_store(qkv, inv_freq, rot, half, self.unit_norm_eps, ctx.pos, ctx.tok_slot, kv, H, G, d, dv,
                                 self.k_dim, self.k_dim, self.v_dim, self.dtype)
-        a = ops.sigmoid_attention(q, kv, ctx.pos, ctx.tok_slot, self.bias, H, G, self.k_dim, dv, self.v_dim,
-                                  self.scale, self.window)
+        if self.dtype == torch.float32:
+            a = ops.sigmoid_attention(q, kv, ctx.pos, ctx.tok_slot, self.bias, H, G, self.k_dim, dv, self.v_dim,
+                                      self.scale, self.window)
+        elif ctx.is_decode:
+            a = ops.sigmoid_attention_decode(q, kv, ctx.seq_slot, ctx.seq_ctx, ctx.n_seqs, self.bias, H, G, self.k_dim,
+                                             dv, self.v_dim, self.scale, self.window, ctx.decode_splits(G, H))
+        else:
+            a = ops.sigmoid_attention_prefill(q, kv, ops.prefill_meta(ctx), self.bias, H, G, self.k_dim, dv,
+                                              self.v_dim, self.scale, self.window)
         return [(ops.linear(a.view(a.shape[0], H * dv), self.wo, out_dtype=torch.float32), 1.0)]
 
     def forward(self, h, ctx, view, residual, owns_cache=True):
