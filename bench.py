@@ -62,10 +62,17 @@ def main() -> int:
                     help="leave out the long contexts, batch 128 and the generation run that the default run adds to points")
     ap.add_argument("--generate", type=int, default=0,
                     help="also generate for this many 128-token prompts with budgets drawn from 16..512 tokens")
+    ap.add_argument("--compare", default="", choices=["", "manirax"],
+                    help="instead of the default workload: prefill and decode throughput of this design at a few "
+                         "layer sizes beside the Llama decoder at equal sizes (random weights, a few layers each)")
+    ap.add_argument("--sizes", default="", help="with --compare: the layer sizes to run, comma separated (default: all)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    if args.compare:
+        print(json.dumps(compare(args)))
+        return 0
 
     if args.shape == "llama-3.1-8b" and not args.no_further_sizes and args.prefill_tokens == 2048:
         args.also_prefill = [16, 128]                      # short prompts, which run as recorded steps
@@ -123,6 +130,102 @@ def main() -> int:
                                             "in 16..512 (greedy, no stop token; tokens/s of the decode phase)").lstrip("; ")
     print(json.dumps(line))
     return 0
+
+
+# layer sizes at which a design is put beside the Llama decoder: width, query heads, key/value heads, head size,
+# feed-forward width, vocabulary
+COMPARE_SIZES = {
+    "2048x16": dict(width=2048, heads=16, kv_heads=4, head_dim=128, ff=8192, vocab=32000),
+    "4096x32": dict(width=4096, heads=32, kv_heads=8, head_dim=128, ff=14336, vocab=32000),
+}
+
+
+def compare_configs(design: str, size: dict, layers: int, context: int) -> dict:
+    """config.json of the design and of the Llama decoder at one size."""
+    w, H, G, hd = size["width"], size["heads"], size["kv_heads"], size["head_dim"]
+    llama = dict(architectures=["LlamaForCausalLM"], num_hidden_layers=layers, hidden_size=w, num_attention_heads=H,
+                 num_key_value_heads=G, head_dim=hd, intermediate_size=size["ff"], vocab_size=size["vocab"],
+                 rope_theta=500000.0, rms_norm_eps=1e-5, max_position_embeddings=context, tie_word_embeddings=True,
+                 hidden_act="silu")
+    assert design == "manirax"
+    # the attention of the same heads beside a linear attention of half as many heads with states of hd x hd
+    layer = {"type": "parallel", "mlp": {"kind": "dense", "ff": size["ff"]},
+             "mixer": {"left": {"heads": H, "kv_heads": G, "dim": hd, "vdim": hd, "scale": hd ** -0.5,
+                                "rot": {"base": 500000.0, "dims": hd // 2, "scaling": {"factor": 4.0}}},
+                       "right": {"heads": H // 2, "dim": hd, "vdim": hd,
+                                 "decay": [1.0 - 2.0 ** -(3 + 5 * i / max(1, H // 2 - 1)) for i in range(H // 2)]},
+                       "left_scale": 0.8, "right_scale": 1.1}}
+    other = {"architecture": "Manirax", "layers": [layer] * layers, "norm": {"eps": 1e-5}, "postln_alpha": 2.5,
+             "vocab": size["vocab"], "width": w, "max_positions": context}
+    return {"llama": llama, design: other}
+
+
+def compare(args) -> dict:
+    """Prefill (one prompt of 512 and of 2,048 tokens) and decode (batch 1, 8 and 32 at a context of 2,048) of
+    the design named and of the Llama decoder, each with 4 layers of the sizes of COMPARE_SIZES."""
+    import gc
+
+    import torch
+
+    import llm_infer_amd
+    from llm_infer_amd.sampling import Sampler
+    layers, context, steps, warmup = args.layers or 4, args.context or 2048, min(args.steps, 32), 4
+    out = {"metric": f"prefill and decode tokens/s, {args.compare} beside llama, {layers} layers", "dtype": args.dtype,
+           "data": "synthetic: random weights, uniform random token ids, cache and states filled with random values",
+           "context": context, "sizes": {}}
+    for size_name, size in COMPARE_SIZES.items():
+        if args.sizes and size_name not in args.sizes.split(","):
+            continue
+        row = out["sizes"][size_name] = {"size": size}
+        for design, raw in compare_configs(args.compare, size, layers, context).items():
+            cfg = llm_infer_amd.config_from_dict(raw)
+            engine = llm_infer_amd.random_model(cfg, seed=0, dtype=args.dtype, max_tokens=33 * (context + 64),
+                                                n_slots=32, same_as_folder=False)
+            cache, res = engine.cache, {}
+            gen = torch.Generator().manual_seed(1)
+            for T in (512, 2048):
+                prompt = torch.randint(0, size["vocab"], (T,), generator=gen).tolist()
+                times = []
+                for _ in range(4):
+                    slot = engine.alloc_slot()
+                    torch.cuda.synchronize()
+                    t = time.perf_counter()
+                    engine.step([slot], [prompt])
+                    torch.cuda.synchronize()
+                    times.append(time.perf_counter() - t)
+                    engine.free_slot(slot)
+                res[f"prefill_{T}_ms"] = round(min(times[1:]) * 1e3, 3)
+                res[f"prefill_{T}_tokens_s"] = round(T / min(times[1:]), 1)
+            for batch in (1, 8, 32):
+                for timed in (False, True):                   # the first walk records the steps
+                    start = context - steps - warmup - 2
+                    slots = [engine.alloc_slot() for _ in range(batch)]
+                    cache.grow(slots, [start] * batch)
+                    for g in cache.groups:
+                        g.storage.normal_(0.0, 1.0)
+                    sampler = Sampler(temperature=0.0, seed=0)
+                    sampler.start(cache, slots, list(range(batch)))
+                    runner = engine.decode_runner(sampler, use_graph=True)
+                    toks = torch.randint(0, size["vocab"], (batch,), generator=gen).tolist()
+                    for _ in range(warmup):
+                        toks = runner.run(slots, toks, may_follow=True)
+                    runner.drain()
+                    torch.cuda.synchronize()
+                    t = time.perf_counter()
+                    for i in range(steps):
+                        toks = runner.run(slots, toks, may_follow=i + 1 < steps)
+                    torch.cuda.synchronize()
+                    dt = time.perf_counter() - t
+                    for sl in slots:
+                        engine.free_slot(sl)
+                res[f"decode_b{batch}_ms"] = round(dt / steps * 1e3, 4)
+                res[f"decode_b{batch}_tokens_s"] = round(batch * steps / dt, 1)
+            row[design] = res
+            print(f"[bench] {size_name} {design}: {res}", file=sys.stderr, flush=True)
+            del engine, cache
+            gc.collect()
+            torch.cuda.empty_cache()
+    return out
 
 
 def measure(args) -> dict:

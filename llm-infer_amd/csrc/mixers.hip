@@ -350,8 +350,13 @@ extern "C" int li_sigmoid_attn(const void* q, void* out, int dt, const void* k_p
 // row groups are added in ascending order through LDS.
 //   proj [T, stride] float32, q at q_off (H heads of d), k at k_off, v at v_off (H heads of dv)
 //   seq_qstart / seq_qlen null: one token per sequence, row i of the step belongs to sequence i (decoding)
+// TR: q, k and v take this type's values after the silu (float: as they are), so that a 16-bit model's
+// decoding multiplies the numbers that its chunked kernel for prompts multiplies.
 // ---------------------------------------------------------------------------
-template <int ROWS>
+template <class T> __device__ __forceinline__ float rounded_to(float v) { return to_f32(from_f32<T>(v)); }
+template <> __device__ __forceinline__ float rounded_to<float>(float v) { return v; }
+
+template <int ROWS, class TR>
 __global__ void decay_attn_kernel(const float* __restrict__ proj, int stride, int q_off, int k_off, int v_off,
                                   float* __restrict__ state, const float* __restrict__ decay,
                                   const int* __restrict__ seq_slot, const int* __restrict__ seq_qstart,
@@ -374,10 +379,10 @@ __global__ void decay_attn_kernel(const float* __restrict__ proj, int stride, in
         const float* row = proj + (int64_t)(q0 + t) * stride;
         __syncthreads();
         for (int i = tid; i < d; i += blockDim.x) {
-            sq[i] = siluf(row[q_off + h * d + i]);
-            sk[i] = siluf(row[k_off + h * d + i]);
+            sq[i] = rounded_to<TR>(siluf(row[q_off + h * d + i]));
+            sk[i] = rounded_to<TR>(siluf(row[k_off + h * d + i]));
         }
-        for (int i = tid; i < dv; i += blockDim.x) sv[i] = siluf(row[v_off + h * dv + i]);
+        for (int i = tid; i < dv; i += blockDim.x) sv[i] = rounded_to<TR>(siluf(row[v_off + h * dv + i]));
         __syncthreads();
         const float vj = sv[j];
         float part = 0.f;
@@ -402,19 +407,268 @@ __global__ void decay_attn_kernel(const float* __restrict__ proj, int stride, in
 
 extern "C" int li_decay_attn(const float* proj, int stride, int q_off, int k_off, int v_off, float* state,
                              const float* decay, const int* seq_slot, const int* seq_qstart, const int* seq_qlen,
-                             float* out, int n_seqs, int H, int d, int dv, hipStream_t stream) {
+                             float* out, int n_seqs, int H, int d, int dv, int round_dt, hipStream_t stream) {
     if (n_seqs <= 0) return LI_OK;
-    if (H <= 0 || d <= 0 || dv <= 0 || dv > 256 || d > 256) return LI_BAD_ARG;
+    if (H <= 0 || d <= 0 || dv <= 0 || dv > 256 || d > 256 || round_dt < DT_F32 || round_dt > DT_BF16) return LI_BAD_ARG;
     int rows = 4;
     while (rows < 64 && ((d + rows - 1) / rows) * dv > 512) rows *= 2;
     const int RG = (d + rows - 1) / rows;
     if (RG * dv > 1024) return LI_UNSUPPORTED;
     dim3 grid(n_seqs, H), block(RG * dv);
     const size_t lds = (size_t)(2 * d + dv + RG * dv) * sizeof(float);
-#define GO(R) decay_attn_kernel<R><<<grid, block, lds, stream>>>(proj, stride, q_off, k_off, v_off, state, decay, \
-        seq_slot, seq_qstart, seq_qlen, out, H, d, dv)
+#define GO1(R, TR) decay_attn_kernel<R, TR><<<grid, block, lds, stream>>>(proj, stride, q_off, k_off, v_off, state, \
+        decay, seq_slot, seq_qstart, seq_qlen, out, H, d, dv)
+#define GO(R) do { if (round_dt == DT_F32) GO1(R, float); else if (round_dt == DT_F16) GO1(R, f16); else GO1(R, bf16); } while (0)
     if (rows == 4) GO(4); else if (rows == 8) GO(8); else if (rows == 16) GO(16); else if (rows == 32) GO(32); else GO(64);
 #undef GO
+#undef GO1
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// The same recurrence for the prompts of a 16-bit model, 32 tokens (a chunk) at a time on the matrix cores.
+// With S the state before a chunk of n tokens, t and s tokens of the chunk, and L = decay[h]:
+//   o_t  = L^(t+1) S^T q_t + sum over s <= t of L^(t-s) (q_t . k_s) v_s
+//   S   <- L^n S + D,   D = sum over s of L^(n-1-s) k_s v_s^T
+// q, k, v are silu of the projections rounded to the 16-bit type T; every product accumulates in float32, and
+// whatever is float32 on its way into a product (the state, the decayed scores, the decayed keys) enters as the
+// sum of two 16-bit numbers, its rounding and the rounding of what is left.  The powers of L are float32.
+// Two kernels.  decay_chunk_kernel, one workgroup per (chunk, head), all chunks of the step at once: the sum
+// within the chunk goes to `out`, D to `ds` [chunk, head, d, dv], and q in 16 bits to `qa` [T, H, 32 DBLK] for the
+// second kernel.  decay_scan_kernel, one workgroup per (sequence, head), walks the sequence's chunks in order:
+// adds L^(t+1) S^T q_t to `out`, then S <- L^n S + D; wave w keeps columns 32w .. 32w+31 of S [d, dv] in
+// accumulator registers (DBLK blocks of 32 rows), so the state is read and written once, and its waves never
+// wait for each other.
+// Accumulator element r of a lane lies at row 8 (r / 4) + 4 (lane / 32) + r % 4 and column lane % 32; an operand
+// whose inner index comes out of an accumulator keeps that order, and the other operand is gathered to match.
+// ---------------------------------------------------------------------------
+template <class T>
+__device__ __forceinline__ void split16(float v, T& hi, T& lo) {
+    hi = from_f32<T>(v);
+    lo = from_f32<T>(v - to_f32(hi));
+}
+
+template <class T, int DBLK, int MAXT>
+__global__ __launch_bounds__(MAXT) void decay_chunk_kernel(
+    const float* __restrict__ proj, int stride, int q_off, int k_off, int v_off, const float* __restrict__ decay,
+    const int* __restrict__ chunk_seq, const int* __restrict__ chunk_t0, const int* __restrict__ seq_qstart,
+    const int* __restrict__ seq_qlen, float* __restrict__ out, float* __restrict__ ds, T* __restrict__ qa, int H, int d,
+    int dv) {
+    typedef typename Vec<T>::v8 v8;
+    constexpr int C = 32, DP = 32 * DBLK, LQ = DP + 8;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int nw = blockDim.x >> 6, LV = 32 * nw + 8;
+    T* sQ = (T*)smem;
+    T* sK = sQ + C * LQ;
+    T* sV = sK + C * LQ;
+    float* pw = (float*)(sV + C * LV);             // pw[i] = L^i, i = 0 .. 32
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, col = lane & 31;
+    const int chunk = blockIdx.x, h = blockIdx.y, seq = chunk_seq[chunk], c0 = chunk_t0[chunk];
+    const int q0 = seq_qstart[seq], nc = min(C, seq_qlen[seq] - c0);
+    const int j = 32 * wave + col;
+    const float lam = decay[h];
+    if (nc <= 0) return;                           // a chunk beyond its sequence's tokens (padding)
+    for (int idx = tid; idx < C * DP; idx += blockDim.x) {
+        const int t = idx / DP, dd = idx - t * DP;
+        float qv = 0.f, kv = 0.f;
+        if (t < nc && dd < d) {
+            const float* row = proj + (int64_t)(q0 + c0 + t) * stride + h * d + dd;
+            qv = siluf(row[q_off]);
+            kv = siluf(row[k_off]);
+        }
+        const T q16 = from_f32<T>(qv);
+        sQ[t * LQ + dd] = q16;
+        sK[t * LQ + dd] = from_f32<T>(kv);
+        if (t < nc) qa[((int64_t)(q0 + c0 + t) * H + h) * DP + dd] = q16;
+    }
+    for (int idx = tid; idx < C * 32 * nw; idx += blockDim.x) {
+        const int t = idx / (32 * nw), jj = idx - t * (32 * nw);
+        float vv = 0.f;
+        if (t < nc && jj < dv) vv = siluf(proj[(int64_t)(q0 + c0 + t) * stride + v_off + h * dv + jj]);
+        sV[t * LV + jj] = from_f32<T>(vv);
+    }
+    if (tid <= C) pw[tid] = powf(lam, (float)tid);
+    __syncthreads();
+    // 1. x[r] = q_t . k_s for s = row(r), t = col, times L^(t-s) where s <= t
+    f32x16 x;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) x[r] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < 2 * DBLK; ++ks) {
+        const v8 a = *(const v8*)(sK + col * LQ + 16 * ks + 8 * half);
+        const v8 b = *(const v8*)(sQ + col * LQ + 16 * ks + 8 * half);
+        x = mfma32(a, b, x);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int s = 8 * (r >> 2) + 4 * half + (r & 3);
+        x[r] = s <= col ? x[r] * pw[col - s] : 0.f;
+    }
+    // 2. within the chunk: o[t, j] = sum over s of w[t, s] v[s, j]   (t = row(r), j = col)
+    f32x16 o;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[r] = 0.f;
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+        v8 whi, wlo, bv;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            T hi, lo;
+            split16<T>(x[8 * u + i], hi, lo);
+            whi[i] = hi; wlo[i] = lo;
+            bv[i] = sV[(16 * u + 8 * (i >> 2) + 4 * half + (i & 3)) * LV + j];
+        }
+        o = mfma32(whi, bv, o);
+        o = mfma32(wlo, bv, o);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int t = 8 * (r >> 2) + 4 * half + (r & 3);
+        if (t < nc && j < dv) out[(int64_t)(q0 + c0 + t) * H * dv + h * dv + j] = o[r];
+    }
+    // 3. D[dd, j] = sum over s of L^(nc-1-s) k[s, dd] v[s, j]
+    float* dst = ds + (((int64_t)chunk * H + h) * d) * dv;
+#pragma unroll
+    for (int blk = 0; blk < DBLK; ++blk) {
+        f32x16 acc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            v8 khi, klo, bv;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int s = 16 * u + 8 * half + i;
+                T hi, lo;
+                split16<T>(s < nc ? pw[nc - 1 - s] * to_f32(sK[s * LQ + 32 * blk + col]) : 0.f, hi, lo);
+                khi[i] = hi; klo[i] = lo;
+                bv[i] = sV[s * LV + j];
+            }
+            acc = mfma32(khi, bv, acc);
+            acc = mfma32(klo, bv, acc);
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int dd = 32 * blk + 8 * (r >> 2) + 4 * half + (r & 3);
+            if (dd < d && j < dv) dst[(int64_t)dd * dv + j] = acc[r];
+        }
+    }
+}
+
+template <class T, int DBLK, int MAXT>
+__global__ __launch_bounds__(MAXT) void decay_scan_kernel(
+    float* __restrict__ state, const float* __restrict__ decay, const int* __restrict__ seq_slot,
+    const int* __restrict__ seq_qstart, const int* __restrict__ seq_qlen, const int* __restrict__ seq_chunk0,
+    float* __restrict__ out, const float* __restrict__ ds, const T* __restrict__ qa, int H, int d, int dv) {
+    typedef typename Vec<T>::v8 v8;
+    typedef typename Vec<T>::v4 v4;
+    constexpr int C = 32, DP = 32 * DBLK;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5, col = lane & 31;
+    const int seq = blockIdx.x, h = blockIdx.y;
+    const int q0 = seq_qstart[seq], n = seq_qlen[seq], chunk0 = seq_chunk0[seq];
+    const int j = 32 * wave + col;
+    const float lam = decay[h];
+    float* Sg = state + (((int64_t)seq_slot[seq] * H + h) * d) * dv;
+    f32x16 S[DBLK];
+    float pwr[16];                                 // L^(t+1) for the rows t of this lane's accumulator elements
+#pragma unroll
+    for (int r = 0; r < 16; ++r) pwr[r] = powf(lam, (float)(8 * (r >> 2) + 4 * half + (r & 3) + 1));
+#pragma unroll
+    for (int blk = 0; blk < DBLK; ++blk)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int dd = 32 * blk + 8 * (r >> 2) + 4 * half + (r & 3);
+            S[blk][r] = (dd < d && j < dv) ? Sg[(int64_t)dd * dv + j] : 0.f;
+        }
+    const float full = powf(lam, (float)C);
+    for (int c0 = 0, c = 0; c0 < n; c0 += C, ++c) {
+        const int nc = min(C, n - c0);
+        // what this chunk brings, asked for before the products that do not need it
+        const float* src = ds + (((int64_t)(chunk0 + c) * H + h) * d) * dv;
+        f32x16 D[DBLK];
+#pragma unroll
+        for (int blk = 0; blk < DBLK; ++blk)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int dd = 32 * blk + 8 * (r >> 2) + 4 * half + (r & 3);
+                D[blk][r] = (dd < d && j < dv) ? src[(int64_t)dd * dv + j] : 0.f;
+            }
+        // o2[t, j] = sum over dd of q[t, dd] S[dd, j]: S in the order its accumulators hold it, q gathered to match
+        const bool row_ok = col < nc;
+        const T* qrow = qa + ((int64_t)(q0 + c0 + (row_ok ? col : 0)) * H + h) * DP + 4 * half;
+        f32x16 o2;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o2[r] = 0.f;
+#pragma unroll
+        for (int blk = 0; blk < DBLK; ++blk)
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                v8 shi, slo, a;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    T hi, lo;
+                    split16<T>(S[blk][8 * u + i], hi, lo);
+                    shi[i] = hi; slo[i] = lo;
+                }
+                v4 a0 = {}, a1 = {};
+                if (row_ok) { a0 = *(const v4*)(qrow + 32 * blk + 16 * u); a1 = *(const v4*)(qrow + 32 * blk + 16 * u + 8); }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) { a[i] = a0[i]; a[4 + i] = a1[i]; }
+                o2 = mfma32(a, shi, o2);
+                o2 = mfma32(a, slo, o2);
+            }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int t = 8 * (r >> 2) + 4 * half + (r & 3);
+            if (t < nc && j < dv) out[(int64_t)(q0 + c0 + t) * H * dv + h * dv + j] += pwr[r] * o2[r];
+        }
+        const float f = nc == C ? full : powf(lam, (float)nc);
+#pragma unroll
+        for (int blk = 0; blk < DBLK; ++blk)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) S[blk][r] = f * S[blk][r] + D[blk][r];
+    }
+#pragma unroll
+    for (int blk = 0; blk < DBLK; ++blk)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int dd = 32 * blk + 8 * (r >> 2) + 4 * half + (r & 3);
+            if (dd < d && j < dv) Sg[(int64_t)dd * dv + j] = S[blk][r];
+        }
+}
+
+// ds: float32 [n_chunks, H, d, dv]; qa: the 16-bit type, [T, H, 32 * ceil(d / 32)]
+extern "C" int li_decay_attn_chunked(const float* proj, int stride, int q_off, int k_off, int v_off, float* state,
+                                     const float* decay, const int* seq_slot, const int* seq_qstart,
+                                     const int* seq_qlen, const int* seq_chunk0, const int* chunk_seq,
+                                     const int* chunk_t0, int n_chunks, float* out, float* ds, void* qa, int n_seqs,
+                                     int H, int d, int dv, int dt, hipStream_t stream) {
+    if (n_seqs <= 0 || n_chunks <= 0) return LI_OK;
+    if (H <= 0 || d <= 0 || dv <= 0 || dv > 256 || d > 256 || !seq_qstart || !seq_qlen || !seq_chunk0 || !chunk_seq ||
+        !chunk_t0 || !ds || !qa)
+        return LI_BAD_ARG;
+    if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
+    const int nw = (dv + 31) / 32, dblk = d <= 32 ? 1 : (d <= 64 ? 2 : (d <= 128 ? 4 : 8));
+    dim3 grid_a(n_chunks, H), grid_b(n_seqs, H), block(64 * nw);
+    const size_t lds = (size_t)(2 * 32 * (32 * dblk + 8) + 32 * (32 * nw + 8)) * 2 + 36 * sizeof(float);
+#define GO2(T, B, M)                                                                                             \
+    do {                                                                                                         \
+        auto kfn = decay_chunk_kernel<T, B, M>;                                                                  \
+        if (lds > 48 * 1024 &&                                                                                   \
+            hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) \
+            return LI_HIP_ERROR;                                                                                 \
+        kfn<<<grid_a, block, lds, stream>>>(proj, stride, q_off, k_off, v_off, decay, chunk_seq, chunk_t0, seq_qstart, \
+                                            seq_qlen, out, ds, (T*)qa, H, d, dv);                                \
+        decay_scan_kernel<T, B, M><<<grid_b, block, 0, stream>>>(state, decay, seq_slot, seq_qstart, seq_qlen,    \
+                                                                 seq_chunk0, out, ds, (const T*)qa, H, d, dv);   \
+    } while (0)
+#define GO1(T, B) do { if (nw <= 4) GO2(T, B, 256); else GO2(T, B, 512); } while (0)
+#define GO(T) do { if (dblk == 1) GO1(T, 1); else if (dblk == 2) GO1(T, 2); else if (dblk == 4) GO1(T, 4); else GO1(T, 8); } while (0)
+    if (dt == DT_F16) GO(f16); else GO(bf16);
+#undef GO
+#undef GO1
+#undef GO2
     LI_CHECK_LAUNCH();
     return LI_OK;
 }

@@ -999,12 +999,39 @@ def sigmoid_attention_decode(q, kv, seq_slot, seq_ctx, n_seqs, bias, n_heads, n_
     return out
 
 
+DECAY_CHUNK = 32        # tokens of one chunk of the chunked decay attention
+
+
+def decay_chunk_lists(qlens) -> tuple:
+    """The chunks of the chunked decay attention for sequences that bring ``qlens`` tokens: for every chunk its
+    sequence and its first token within the sequence's tokens, and for every sequence its first chunk."""
+    chunk_seq, chunk_t0, seq_chunk0 = [], [], []
+    for i, n in enumerate(qlens):
+        seq_chunk0.append(len(chunk_seq))
+        for t0 in range(0, n, DECAY_CHUNK):
+            chunk_seq.append(i)
+            chunk_t0.append(t0)
+    return chunk_seq, chunk_t0, seq_chunk0
+
+
+def decay_chunks(ctx) -> dict:
+    """The chunk lists of a step on the device, made and uploaded once per step by the first layer that asks."""
+    def make():
+        chunk_seq, chunk_t0, seq_chunk0 = decay_chunk_lists(ctx.host_qlens)
+        flat = torch.tensor(chunk_seq + chunk_t0 + seq_chunk0, dtype=torch.int32).to(ctx.device)
+        n = len(chunk_seq)
+        return {"chunk_seq": flat[:n], "chunk_t0": flat[n:2 * n], "seq_chunk0": flat[2 * n:], "n_chunks": n}
+    return ctx.shared(("decay_attention_chunks", DECAY_CHUNK), make)
+
+
 def decay_attention(proj, q_off, k_off, v_off, state, decay, seq_slot, seq_qstart, seq_qlen, n_seqs, n_heads,
-                    head_dim, v_head_dim) -> torch.Tensor:
+                    head_dim, v_head_dim, round_to=None, chunked: bool = False, chunks=None) -> torch.Tensor:
     """Linear attention with a constant decay per head over the tokens of a step, from and into the float32
     ``state`` [slots, H, d, dv]: S <- decay S + k v^T, o = S^T q, with q, k, v = silu of the columns of ``proj``
     (float32 [T, n]) at the given offsets.  ``seq_qstart`` / ``seq_qlen`` None: one token per sequence.
-    Returns float32 [T, H * dv]."""
+    ``round_to`` (a 16-bit type): q, k and v take that type's values after the silu.  ``chunked`` (needs
+    ``round_to``, the per-sequence arrays and ``chunks`` = ``decay_chunks(ctx)``): 32 tokens at a time on the
+    matrix cores, for prompts; else token by token.  Returns float32 [T, H * dv]."""
     _dev(proj, state, decay, seq_slot, seq_qstart, seq_qlen)
     _f32_rows(proj, "decay_attention proj")
     H, d, dv = n_heads, head_dim, v_head_dim
@@ -1017,10 +1044,23 @@ def decay_attention(proj, q_off, k_off, v_off, state, decay, seq_slot, seq_qstar
     else:
         _need(seq_qlen is not None and seq_qstart.dtype == torch.int32 and seq_qlen.dtype == torch.int32 and
               seq_qstart.numel() >= n_seqs and seq_qlen.numel() >= n_seqs, "seq_qstart, seq_qlen: int32 [sequences]")
+    _need(round_to in (None, torch.float32, torch.float16, torch.bfloat16), "round_to: a 16-bit type or None")
     out = torch.empty((proj.shape[0], H * dv), dtype=torch.float32, device=proj.device)
+    if chunked:
+        _need(round_to in (torch.float16, torch.bfloat16) and seq_qstart is not None and chunks is not None,
+              "the chunked kernels multiply 16-bit numbers and need the sequences' rows and the list of chunks")
+        n_chunks = chunks["n_chunks"]
+        ds = torch.empty((max(1, n_chunks), H, d, dv), dtype=torch.float32, device=proj.device)
+        qa = torch.empty((proj.shape[0], H, (d + 31) // 32 * 32), dtype=round_to, device=proj.device)
+        _check(mixers().li_decay_attn_chunked(_ptr(proj), proj.shape[1], q_off, k_off, v_off, _ptr(state), _ptr(decay),
+                                              _ptr(seq_slot), _ptr(seq_qstart), _ptr(seq_qlen), _ptr(chunks["seq_chunk0"]),
+                                              _ptr(chunks["chunk_seq"]), _ptr(chunks["chunk_t0"]), n_chunks, _ptr(out),
+                                              _ptr(ds), _ptr(qa), n_seqs, H, d, dv, DT[round_to], _stream()),
+               "decay_attn_chunked")
+        return out
     _check(mixers().li_decay_attn(_ptr(proj), proj.shape[1], q_off, k_off, v_off, _ptr(state), _ptr(decay),
                                   _ptr(seq_slot), _ptr(seq_qstart), _ptr(seq_qlen), _ptr(out), n_seqs, H, d, dv,
-                                  _stream()), "decay_attn")
+                                  DT[round_to or torch.float32], _stream()), "decay_attn")
     return out
 
 
