@@ -83,12 +83,68 @@ __global__ void add_layernorm_kernel(float* __restrict__ x, float alpha, const f
     }
 }
 
+// The same for rows of up to N * blockDim.x elements: a thread keeps its N elements in registers, so the row is
+// read once and written once.
+template <class TC, int N>
+__global__ __launch_bounds__(1024) void add_layernorm_reg_kernel(float* __restrict__ x, float alpha, const float* __restrict__ y1, float s1,
+                                         const float* __restrict__ y2, float s2, const float* __restrict__ w, float eps,
+                                         TC* __restrict__ copy, int d) {
+    __shared__ float scratch[16];
+    const int64_t base = (int64_t)blockIdx.x * d;
+    float v[N];
+    float s = 0.f;
+#pragma unroll
+    for (int u = 0; u < N; ++u) {
+        const int i = threadIdx.x + u * blockDim.x;
+        v[u] = 0.f;
+        if (i < d) {
+            float y = s1 * y1[base + i];
+            if (y2) y += s2 * y2[base + i];
+            v[u] = alpha * x[base + i] + y;
+            s += v[u];
+        }
+    }
+    const float mean = block_sum(s, scratch) / (float)d;
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < N; ++u) {
+        const int i = threadIdx.x + u * blockDim.x;
+        if (i < d) { v[u] -= mean; ss += v[u] * v[u]; }
+    }
+    const float sd = sqrtf(block_sum(ss, scratch) / (float)d + eps);
+#pragma unroll
+    for (int u = 0; u < N; ++u) {
+        const int i = threadIdx.x + u * blockDim.x;
+        if (i < d) {
+            const float r = v[u] / sd * w[i];
+            x[base + i] = r;
+            if (copy) copy[base + i] = from_f32<TC>(r);
+        }
+    }
+}
+
 extern "C" int li_add_layernorm(float* x, float alpha, const float* y1, float s1, const float* y2, float s2,
                                 const float* w, float eps, void* copy, int copy_dt, int n_rows, int d,
                                 hipStream_t stream) {
     if (n_rows <= 0) return LI_OK;
     if (d <= 0 || !y1) return LI_BAD_ARG;
     dim3 grid(n_rows), block(d >= 2048 ? 512 : (d >= 256 ? 256 : 64));
+    if (d <= 8 * 1024) {
+        const int per = d <= 4096 ? 4 : 8;
+        dim3 rb(((d + per - 1) / per + 63) / 64 * 64);
+#define GO(TC)                                                                                                        \
+    do {                                                                                                              \
+        if (per == 4) add_layernorm_reg_kernel<TC, 4><<<grid, rb, 0, stream>>>(x, alpha, y1, s1, y2, s2, w, eps, (TC*)copy, d); \
+        else add_layernorm_reg_kernel<TC, 8><<<grid, rb, 0, stream>>>(x, alpha, y1, s1, y2, s2, w, eps, (TC*)copy, d);        \
+    } while (0)
+        if (!copy || copy_dt == DT_F32) GO(float);
+        else if (copy_dt == DT_F16) GO(f16);
+        else if (copy_dt == DT_BF16) GO(bf16);
+        else return LI_BAD_ARG;
+#undef GO
+        LI_CHECK_LAUNCH();
+        return LI_OK;
+    }
     if (!copy || copy_dt == DT_F32)
         add_layernorm_kernel<float><<<grid, block, 0, stream>>>(x, alpha, y1, s1, y2, s2, w, eps, (float*)copy, d);
     else if (copy_dt == DT_F16)
@@ -142,19 +198,23 @@ extern "C" int li_cast(const float* x, void* out, int out_dt, int64_t n, hipStre
 // kernel then leaves each sequence's last row of this step in its state.  The rows of one sequence are
 // consecutive and no two sequences share a slot, so a change of tok_slot marks a sequence's edge.
 // ---------------------------------------------------------------------------
+// `single`: every sequence brings one row (decoding), so each row is its sequence's first and last; the thread
+// that has read an element of the state then writes the row's own element there, and no second kernel runs.
 template <class TO>
 __global__ void token_shift_kernel(const float* __restrict__ x, const float* __restrict__ mu,
-                                   const float* __restrict__ state, const int* __restrict__ pos,
-                                   const int* __restrict__ tok_slot, TO* __restrict__ out, int d) {
+                                   float* __restrict__ state, const int* __restrict__ pos,
+                                   const int* __restrict__ tok_slot, TO* __restrict__ out, int d, int single) {
     const int t = blockIdx.x;
     const int slot = tok_slot[t];
-    const bool first = t == 0 || tok_slot[t - 1] != slot;
-    const float* prev = pos[t] == 0 ? nullptr : (first ? state + (int64_t)slot * d : x + (int64_t)(t - 1) * d);
+    const bool first = single || t == 0 || tok_slot[t - 1] != slot;
+    float* st = state + (int64_t)slot * d;
+    const float* prev = pos[t] == 0 ? nullptr : (first ? st : x + (int64_t)(t - 1) * d);
     const float* xr = x + (int64_t)t * d;
     TO* o = out + (int64_t)t * d;
     for (int i = threadIdx.x; i < d; i += blockDim.x) {
         const float h = xr[i], p = prev ? prev[i] : 0.f;
         o[i] = from_f32<TO>(h + (p - h) * mu[i]);
+        if (single) st[i] = h;
     }
 }
 
@@ -169,15 +229,16 @@ __global__ void token_shift_save_kernel(const float* __restrict__ x, float* __re
 }
 
 extern "C" int li_token_shift(const float* x, const float* mu, float* state, const int* pos, const int* tok_slot,
-                              void* out, int out_dt, int n_tokens, int d, hipStream_t stream) {
+                              void* out, int out_dt, int n_tokens, int d, int single, hipStream_t stream) {
     if (n_tokens <= 0) return LI_OK;
     if (d <= 0) return LI_BAD_ARG;
     dim3 grid(n_tokens), block(d >= 1024 ? 256 : 64);
-    if (out_dt == DT_F32) token_shift_kernel<float><<<grid, block, 0, stream>>>(x, mu, state, pos, tok_slot, (float*)out, d);
-    else if (out_dt == DT_F16) token_shift_kernel<f16><<<grid, block, 0, stream>>>(x, mu, state, pos, tok_slot, (f16*)out, d);
-    else if (out_dt == DT_BF16) token_shift_kernel<bf16><<<grid, block, 0, stream>>>(x, mu, state, pos, tok_slot, (bf16*)out, d);
+    if (out_dt == DT_F32) token_shift_kernel<float><<<grid, block, 0, stream>>>(x, mu, state, pos, tok_slot, (float*)out, d, single);
+    else if (out_dt == DT_F16) token_shift_kernel<f16><<<grid, block, 0, stream>>>(x, mu, state, pos, tok_slot, (f16*)out, d, single);
+    else if (out_dt == DT_BF16) token_shift_kernel<bf16><<<grid, block, 0, stream>>>(x, mu, state, pos, tok_slot, (bf16*)out, d, single);
     else return LI_BAD_ARG;
     LI_CHECK_LAUNCH();
+    if (single) return LI_OK;
     token_shift_save_kernel<<<grid, block, 0, stream>>>(x, state, tok_slot, d, n_tokens);
     LI_CHECK_LAUNCH();
     return LI_OK;
@@ -205,7 +266,7 @@ __global__ __launch_bounds__(256) void rope_norm_store_kernel(
     int64_t page = 0;
     if (G > 0) page = c.page_table[(int64_t)tok_slot[t] * c.max_pages + p / PAGE];
     const int tp = p % PAGE, half = rot >> 1;
-    for (int head = wave; head < H + 2 * G; head += n_waves) {
+    for (int head = blockIdx.y * n_waves + wave; head < H + 2 * G; head += n_waves * gridDim.y) {
         if (head < H + G) {
             const float* src = row + (int64_t)head * d;
             float val[4];
@@ -264,7 +325,8 @@ extern "C" int li_rope_norm_store(const float* qkv, int row_stride, const float*
     if (G > 0 && (dv <= 0 || dk < d || dk > 256 || dk % 16 || dvp < dv || dvp % 16 || !page_table)) return LI_BAD_ARG;
     if (row_stride < (H + G) * d + G * dv || (rot > 0 && !inv_freq)) return LI_BAD_ARG;
     Pages c{k_pages, v_pages, page_stride, page_table, max_pages};
-    dim3 grid(n_tokens), block(256);
+    // few tokens: the heads spread over the grid as well
+    dim3 grid(n_tokens, n_tokens >= 512 ? 1 : (H + 2 * G + 3) / 4), block(256);
 #define GO(T) rope_norm_store_kernel<T><<<grid, block, 0, stream>>>(qkv, row_stride, inv_freq, rot, half_pairing, \
         unit_eps, pos, tok_slot, c, (T*)q_out, H, G, d, dv, dq, dk, dvp)
     if (dt == DT_F32) GO(float); else if (dt == DT_F16) GO(f16); else if (dt == DT_BF16) GO(bf16); else return LI_BAD_ARG;
@@ -434,12 +496,11 @@ extern "C" int li_decay_attn(const float* proj, int stride, int q_off, int k_off
 // q, k, v are silu of the projections rounded to the 16-bit type T; every product accumulates in float32, and
 // whatever is float32 on its way into a product (the state, the decayed scores, the decayed keys) enters as the
 // sum of two 16-bit numbers, its rounding and the rounding of what is left.  The powers of L are float32.
-// Two kernels.  decay_chunk_kernel, one workgroup per (chunk, head), all chunks of the step at once: the sum
-// within the chunk goes to `out`, D to `ds` [chunk, head, d, dv], and q in 16 bits to `qa` [T, H, 32 DBLK] for the
-// second kernel.  decay_scan_kernel, one workgroup per (sequence, head), walks the sequence's chunks in order:
-// adds L^(t+1) S^T q_t to `out`, then S <- L^n S + D; wave w keeps columns 32w .. 32w+31 of S [d, dv] in
-// accumulator registers (DBLK blocks of 32 rows), so the state is read and written once, and its waves never
-// wait for each other.
+// Three kernels, of which only the middle one walks a sequence in order.  decay_chunk_kernel, one workgroup per
+// (chunk, head), all chunks of the step at once: the sum within the chunk goes to `out`, D to `ds` [chunk, head,
+// d, dv], and q in 16 bits to `qa` [T, H, 32 DBLK].  decay_scan_kernel, a thread per element of S: the states
+// before every chunk, left where the D were.  decay_carry_kernel, again one workgroup per (chunk, head): adds
+// L^(t+1) S^T q_t to `out`.
 // Accumulator element r of a lane lies at row 8 (r / 4) + 4 (lane / 32) + r % 4 and column lane % 32; an operand
 // whose inner index comes out of an accumulator keeps that order, and the other operand is gathered to match.
 // ---------------------------------------------------------------------------
@@ -556,86 +617,75 @@ __global__ __launch_bounds__(MAXT) void decay_chunk_kernel(
     }
 }
 
+// The states before every chunk, element by element: thread e of (sequence, head) walks the sequence's chunks
+// in order, leaves the state before chunk c where D_c was, and goes on with S <- L^n S + D_c.
+__global__ void decay_scan_kernel(float* __restrict__ state, const float* __restrict__ decay,
+                                  const int* __restrict__ seq_slot, const int* __restrict__ seq_qlen,
+                                  const int* __restrict__ seq_chunk0, float* __restrict__ ds, int H, int d, int dv) {
+    constexpr int C = 32;
+    const int seq = blockIdx.y, h = blockIdx.z;
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x, per = (int64_t)d * dv;
+    if (e >= per) return;
+    const int n = seq_qlen[seq];
+    const float lam = decay[h], full = powf(lam, (float)C);
+    float* Sg = state + ((int64_t)seq_slot[seq] * H + h) * per + e;
+    float* p = ds + ((int64_t)seq_chunk0[seq] * H + h) * per + e;
+    float S = *Sg;
+    for (int c0 = 0; c0 < n; c0 += C, p += (int64_t)H * per) {
+        const float D = *p;
+        *p = S;
+        S = (n - c0 >= C ? full : powf(lam, (float)(n - c0))) * S + D;
+    }
+    *Sg = S;
+}
+
+// out[t, j] += L^(t+1) sum over dd of q[t, dd] S[dd, j] for the tokens of one chunk, S the state before the chunk
+// (what decay_scan_kernel left in `ds`): one workgroup per (chunk, head), wave w the columns 32w .. 32w+31.  S is
+// read in the order in which accumulators hold their rows and q gathered to match.
 template <class T, int DBLK, int MAXT>
-__global__ __launch_bounds__(MAXT) void decay_scan_kernel(
-    float* __restrict__ state, const float* __restrict__ decay, const int* __restrict__ seq_slot,
-    const int* __restrict__ seq_qstart, const int* __restrict__ seq_qlen, const int* __restrict__ seq_chunk0,
-    float* __restrict__ out, const float* __restrict__ ds, const T* __restrict__ qa, int H, int d, int dv) {
+__global__ __launch_bounds__(MAXT) void decay_carry_kernel(
+    const float* __restrict__ decay, const int* __restrict__ chunk_seq, const int* __restrict__ chunk_t0,
+    const int* __restrict__ seq_qstart, const int* __restrict__ seq_qlen, float* __restrict__ out,
+    const float* __restrict__ ds, const T* __restrict__ qa, int H, int d, int dv) {
     typedef typename Vec<T>::v8 v8;
     typedef typename Vec<T>::v4 v4;
     constexpr int C = 32, DP = 32 * DBLK;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5, col = lane & 31;
-    const int seq = blockIdx.x, h = blockIdx.y;
-    const int q0 = seq_qstart[seq], n = seq_qlen[seq], chunk0 = seq_chunk0[seq];
+    const int chunk = blockIdx.x, h = blockIdx.y, seq = chunk_seq[chunk], c0 = chunk_t0[chunk];
+    const int q0 = seq_qstart[seq], nc = min(C, seq_qlen[seq] - c0);
+    if (nc <= 0) return;
     const int j = 32 * wave + col;
     const float lam = decay[h];
-    float* Sg = state + (((int64_t)seq_slot[seq] * H + h) * d) * dv;
-    f32x16 S[DBLK];
-    float pwr[16];                                 // L^(t+1) for the rows t of this lane's accumulator elements
+    const float* src = ds + (((int64_t)chunk * H + h) * d) * dv;
+    const bool row_ok = col < nc;
+    const T* qrow = qa + ((int64_t)(q0 + c0 + (row_ok ? col : 0)) * H + h) * DP + 4 * half;
+    f32x16 o2;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) pwr[r] = powf(lam, (float)(8 * (r >> 2) + 4 * half + (r & 3) + 1));
+    for (int r = 0; r < 16; ++r) o2[r] = 0.f;
 #pragma unroll
     for (int blk = 0; blk < DBLK; ++blk)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int dd = 32 * blk + 8 * (r >> 2) + 4 * half + (r & 3);
-            S[blk][r] = (dd < d && j < dv) ? Sg[(int64_t)dd * dv + j] : 0.f;
-        }
-    const float full = powf(lam, (float)C);
-    for (int c0 = 0, c = 0; c0 < n; c0 += C, ++c) {
-        const int nc = min(C, n - c0);
-        // what this chunk brings, asked for before the products that do not need it
-        const float* src = ds + (((int64_t)(chunk0 + c) * H + h) * d) * dv;
-        f32x16 D[DBLK];
+        for (int u = 0; u < 2; ++u) {
+            v8 shi, slo, a;
 #pragma unroll
-        for (int blk = 0; blk < DBLK; ++blk)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int dd = 32 * blk + 8 * (r >> 2) + 4 * half + (r & 3);
-                D[blk][r] = (dd < d && j < dv) ? src[(int64_t)dd * dv + j] : 0.f;
+            for (int i = 0; i < 8; ++i) {
+                const int dd = 32 * blk + 16 * u + 8 * (i >> 2) + 4 * half + (i & 3);
+                T hi, lo;
+                split16<T>((dd < d && j < dv) ? src[(int64_t)dd * dv + j] : 0.f, hi, lo);
+                shi[i] = hi; slo[i] = lo;
             }
-        // o2[t, j] = sum over dd of q[t, dd] S[dd, j]: S in the order its accumulators hold it, q gathered to match
-        const bool row_ok = col < nc;
-        const T* qrow = qa + ((int64_t)(q0 + c0 + (row_ok ? col : 0)) * H + h) * DP + 4 * half;
-        f32x16 o2;
+            v4 a0 = {}, a1 = {};
+            if (row_ok) { a0 = *(const v4*)(qrow + 32 * blk + 16 * u); a1 = *(const v4*)(qrow + 32 * blk + 16 * u + 8); }
 #pragma unroll
-        for (int r = 0; r < 16; ++r) o2[r] = 0.f;
-#pragma unroll
-        for (int blk = 0; blk < DBLK; ++blk)
-#pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                v8 shi, slo, a;
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    T hi, lo;
-                    split16<T>(S[blk][8 * u + i], hi, lo);
-                    shi[i] = hi; slo[i] = lo;
-                }
-                v4 a0 = {}, a1 = {};
-                if (row_ok) { a0 = *(const v4*)(qrow + 32 * blk + 16 * u); a1 = *(const v4*)(qrow + 32 * blk + 16 * u + 8); }
-#pragma unroll
-                for (int i = 0; i < 4; ++i) { a[i] = a0[i]; a[4 + i] = a1[i]; }
-                o2 = mfma32(a, shi, o2);
-                o2 = mfma32(a, slo, o2);
-            }
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int t = 8 * (r >> 2) + 4 * half + (r & 3);
-            if (t < nc && j < dv) out[(int64_t)(q0 + c0 + t) * H * dv + h * dv + j] += pwr[r] * o2[r];
+            for (int i = 0; i < 4; ++i) { a[i] = a0[i]; a[4 + i] = a1[i]; }
+            o2 = mfma32(a, shi, o2);
+            o2 = mfma32(a, slo, o2);
         }
-        const float f = nc == C ? full : powf(lam, (float)nc);
 #pragma unroll
-        for (int blk = 0; blk < DBLK; ++blk)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) S[blk][r] = f * S[blk][r] + D[blk][r];
+    for (int r = 0; r < 16; ++r) {
+        const int t = 8 * (r >> 2) + 4 * half + (r & 3);
+        if (t < nc && j < dv) out[(int64_t)(q0 + c0 + t) * H * dv + h * dv + j] += powf(lam, (float)(t + 1)) * o2[r];
     }
-#pragma unroll
-    for (int blk = 0; blk < DBLK; ++blk)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int dd = 32 * blk + 8 * (r >> 2) + 4 * half + (r & 3);
-            if (dd < d && j < dv) Sg[(int64_t)dd * dv + j] = S[blk][r];
-        }
 }
 
 // ds: float32 [n_chunks, H, d, dv]; qa: the 16-bit type, [T, H, 32 * ceil(d / 32)]
@@ -650,7 +700,7 @@ extern "C" int li_decay_attn_chunked(const float* proj, int stride, int q_off, i
         return LI_BAD_ARG;
     if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
     const int nw = (dv + 31) / 32, dblk = d <= 32 ? 1 : (d <= 64 ? 2 : (d <= 128 ? 4 : 8));
-    dim3 grid_a(n_chunks, H), grid_b(n_seqs, H), block(64 * nw);
+    dim3 grid_a(n_chunks, H), block(64 * nw);
     const size_t lds = (size_t)(2 * 32 * (32 * dblk + 8) + 32 * (32 * nw + 8)) * 2 + 36 * sizeof(float);
 #define GO2(T, B, M)                                                                                             \
     do {                                                                                                         \
@@ -660,8 +710,10 @@ extern "C" int li_decay_attn_chunked(const float* proj, int stride, int q_off, i
             return LI_HIP_ERROR;                                                                                 \
         kfn<<<grid_a, block, lds, stream>>>(proj, stride, q_off, k_off, v_off, decay, chunk_seq, chunk_t0, seq_qstart, \
                                             seq_qlen, out, ds, (T*)qa, H, d, dv);                                \
-        decay_scan_kernel<T, B, M><<<grid_b, block, 0, stream>>>(state, decay, seq_slot, seq_qstart, seq_qlen,    \
-                                                                 seq_chunk0, out, ds, (const T*)qa, H, d, dv);   \
+        decay_scan_kernel<<<dim3((d * dv + 255) / 256, n_seqs, H), 256, 0, stream>>>(state, decay, seq_slot, seq_qlen, \
+                                                                                    seq_chunk0, ds, H, d, dv);    \
+        decay_carry_kernel<T, B, M><<<grid_a, block, 0, stream>>>(decay, chunk_seq, chunk_t0, seq_qstart, seq_qlen, out, \
+                                                                  ds, (const T*)qa, H, d, dv);                    \
     } while (0)
 #define GO1(T, B) do { if (nw <= 4) GO2(T, B, 256); else GO2(T, B, 512); } while (0)
 #define GO(T) do { if (dblk == 1) GO1(T, 1); else if (dblk == 2) GO1(T, 2); else if (dblk == 4) GO1(T, 4); else GO1(T, 8); } while (0)
@@ -730,11 +782,49 @@ __global__ void polynorm_kernel(const float* __restrict__ z, const float* __rest
     }
 }
 
+// The same for rows of up to 16 * blockDim.x elements, read once and kept in registers.
+template <class TO>
+__global__ void polynorm_reg_kernel(const float* __restrict__ z, const float* __restrict__ coef, TO* __restrict__ out,
+                                    int n, float eps) {
+    __shared__ float scratch[16];
+    const int64_t base = (int64_t)blockIdx.x * n;
+    float v[16];
+    float s1 = 0.f, s2 = 0.f, s3 = 0.f;
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+        const int i = threadIdx.x + u * blockDim.x;
+        v[u] = i < n ? z[base + i] : 0.f;
+        const float v2 = v[u] * v[u], v3 = v2 * v[u];
+        s1 += v2; s2 += v2 * v2; s3 += v3 * v3;
+    }
+    const float r1 = sqrtf(block_sum(s1, scratch) / (float)n + eps);
+    const float r2 = sqrtf(block_sum(s2, scratch) / (float)n + eps);
+    const float r3 = sqrtf(block_sum(s3, scratch) / (float)n + eps);
+    const float a = coef[0], b = coef[1], c = coef[2], e = coef[3];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+        const int i = threadIdx.x + u * blockDim.x;
+        if (i < n) {
+            const float v2 = v[u] * v[u], v3 = v2 * v[u];
+            out[base + i] = from_f32<TO>(a * (v[u] / r1) + b * (v2 / r2) + c * (v3 / r3) + e);
+        }
+    }
+}
+
 extern "C" int li_polynorm(const float* z, const float* coef, void* out, int out_dt, int n_rows, int n, float eps,
                            hipStream_t stream) {
     if (n_rows <= 0) return LI_OK;
     if (n <= 0) return LI_BAD_ARG;
     dim3 grid(n_rows), block(n >= 2048 ? 512 : (n >= 256 ? 256 : 64));
+    if (n <= 16 * 1024) {
+        dim3 rb(n <= 1024 ? 64 : (n <= 4096 ? 256 : (n <= 8192 ? 512 : 1024)));
+        if (out_dt == DT_F32) polynorm_reg_kernel<float><<<grid, rb, 0, stream>>>(z, coef, (float*)out, n, eps);
+        else if (out_dt == DT_F16) polynorm_reg_kernel<f16><<<grid, rb, 0, stream>>>(z, coef, (f16*)out, n, eps);
+        else if (out_dt == DT_BF16) polynorm_reg_kernel<bf16><<<grid, rb, 0, stream>>>(z, coef, (bf16*)out, n, eps);
+        else return LI_BAD_ARG;
+        LI_CHECK_LAUNCH();
+        return LI_OK;
+    }
     if (out_dt == DT_F32) polynorm_kernel<float><<<grid, block, 0, stream>>>(z, coef, (float*)out, n, eps);
     else if (out_dt == DT_F16) polynorm_kernel<f16><<<grid, block, 0, stream>>>(z, coef, (f16*)out, n, eps);
     else if (out_dt == DT_BF16) polynorm_kernel<bf16><<<grid, block, 0, stream>>>(z, coef, (bf16*)out, n, eps);

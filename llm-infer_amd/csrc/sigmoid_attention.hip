@@ -9,7 +9,8 @@
 // page in operand order (common.h), one contiguous 1 KiB load per fragment.  Scores and weights are float32;
 // a weight goes into the second product as the sum of two 16-bit numbers (its rounding and the rounding of
 // what is left), so that the product sees 16 bits of it and not 8.
-//   prompt : a workgroup is 4 waves = 128 consecutive tokens of one sequence and one query head
+//   prompt : a workgroup is 4 waves = 128 consecutive tokens of one sequence and one query head; a page is
+//            fetched once for the four, through two stages of LDS
 //   decode : one wave per (sequence, key/value head, split of the context); with more than one split the
 //            partial sums are added in ascending order by a second kernel
 #include "common.h"
@@ -69,11 +70,14 @@ struct WaveSigmoid {
                                             float bias2, bool masked) {
         const int lane = threadIdx.x & 63;
 #pragma unroll
-        for (int b = 0; b < 2; ++b) {
+        for (int b = 0; b < 2; ++b)
 #pragma unroll
             for (int r = 0; r < 16; ++r) s[b][r] = 0.f;
+        // the two blocks of keys in turn, so that no matrix instruction waits for the one before it
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) s[b] = mfma32(kf[b * KS + ks], q[ks], s[b]);
+        for (int ks = 0; ks < KS; ++ks) {
+            s[0] = mfma32(kf[ks], q[ks], s[0]);
+            s[1] = mfma32(kf[KS + ks], q[ks], s[1]);
         }
 #pragma unroll
         for (int b = 0; b < 2; ++b)
@@ -100,10 +104,9 @@ struct WaveSigmoid {
                 lo[i] = from_f32<T>(w - to_f32(hi[i]));
             }
 #pragma unroll
-            for (int b = 0; b < DB; ++b) {
-                o[b] = mfma32(vf[b * 4 + tj], hi, o[b]);
-                o[b] = mfma32(vf[b * 4 + tj], lo, o[b]);
-            }
+            for (int b = 0; b < DB; ++b) o[b] = mfma32(vf[b * 4 + tj], hi, o[b]);
+#pragma unroll
+            for (int b = 0; b < DB; ++b) o[b] = mfma32(vf[b * 4 + tj], lo, o[b]);
         }
     }
 };
@@ -118,11 +121,22 @@ __global__ __launch_bounds__(256) void sigmoid_prefill_kernel(
     const int* __restrict__ tile_q0, const int* __restrict__ seq_slot, const int* __restrict__ seq_qstart,
     const int* __restrict__ seq_qlen, const int* __restrict__ seq_ctx, const float* __restrict__ bias, int H, int G,
     int dv, float scale, int window) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, row = lane & 31;
-    const int seq = tile_seq[blockIdx.x], h = blockIdx.y, g = h / (H / G);
-    const int qlen = seq_qlen[seq], q0 = tile_q0[blockIdx.x] + 32 * wave;
-    if (q0 >= qlen) return;
-    const int before = seq_ctx[seq] - qlen;                 // the sequence's tokens before this step
+    typedef typename WaveSigmoid<T>::v8 v8;
+    constexpr int KE = PAGE * KD, VE = PAGE * DB * 32;        // elements of one head's keys and values in a page
+    constexpr int KN = KE / 8, KP = (KN + 255) / 256, VP = VE / (256 * 8);   // 16-byte pieces: of the keys, and a thread's
+    static_assert(VE % (256 * 8) == 0, "the values of a page divide among the workgroup's threads");
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    T* smem = (T*)smem_raw;                                   // two stages of [keys | values]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, row = lane & 31;
+    // workgroups start in the order of their number: the last tiles of a prompt, which see the most keys, go
+    // first and all heads of a tile together, so that the short ones fill the chip's tail
+    const int number = blockIdx.x + gridDim.x * blockIdx.y;
+    const int tile = gridDim.x - 1 - number / H, h = number % H, g = h / (H / G);
+    const int seq = tile_seq[tile];
+    const int qlen = seq_qlen[seq], tile0 = tile_q0[tile], q0 = tile0 + 32 * wave;
+    if (tile0 >= qlen) return;                                // the whole workgroup: a tile of padding
+    const bool active = q0 < qlen;                            // a wave without tokens still helps to fetch
+    const int before = seq_ctx[seq] - qlen;                   // the sequence's tokens before this step
     const bool valid = q0 + row < qlen;
     const int64_t tok = (int64_t)seq_qstart[seq] + q0 + row;
     const int pos = before + q0 + row;
@@ -132,20 +146,52 @@ __global__ __launch_bounds__(256) void sigmoid_prefill_kernel(
     const int pos_min = before + q0, pos_max = before + min(q0 + 31, qlen - 1);
     const int lo_min = window > 0 ? max(0, pos_min - window + 1) : 0, lo_max = window > 0 ? max(0, pos_max - window + 1) : 0;
     const bool all_valid = q0 + 31 < qlen;
-    const int p0 = lo_min / PAGE, p1 = pos_max / PAGE + 1;
+    const int p0 = lo_min / PAGE, p1 = active ? pos_max / PAGE + 1 : 0;          // this wave's pages
+    // the workgroup's pages: from the first page of its first token to the last page of its last
+    const int wg_first = before + tile0, wg_last = before + min(tile0 + 127, qlen - 1);
+    const int P0 = (window > 0 ? max(0, wg_first - window + 1) : 0) / PAGE, P1 = wg_last / PAGE + 1;
     const int* table = c.page_table + (int64_t)seq_slot[seq] * c.max_pages;
     const float scale2 = scale * LOG2E, bias2 = (bias ? bias[h] : 0.f) * LOG2E;
-    typename WaveSigmoid<T>::v8 kf[2 * KS], vf[DB * 4];
-    f32x16 s[2];
     const T* kbase = (const T*)c.k + (int64_t)g * k_head_elems(KD);
     const T* vbase = (const T*)c.v + (int64_t)g * v_head_elems(VD);
-    a.load_k(kbase + (int64_t)table[p0] * c.page_stride, kf);
-    for (int p = p0; p < p1; ++p) {
-        a.load_v(vbase + (int64_t)table[p] * c.page_stride, vf);
-        const bool inside = all_valid && p * PAGE >= lo_max && p * PAGE + PAGE - 1 <= pos_min;
-        a.weights(kf, s, p * PAGE, lo, hi, scale2, bias2, !inside);
-        if (p + 1 < p1) a.load_k(kbase + (int64_t)table[p + 1] * c.page_stride, kf);
-        a.mix(vf, s);
+    // A page is fetched once for the four waves: every thread brings 16-byte pieces of it into registers while
+    // the page before is worked on, and lays them into the other stage of LDS afterwards; one barrier a page.
+    v8 rk[KP], rv[VP];
+    auto fetch = [&](int p) {
+        const T* kp = kbase + (int64_t)table[p] * c.page_stride;
+        const T* vp = vbase + (int64_t)table[p] * c.page_stride;
+#pragma unroll
+        for (int i = 0; i < KP; ++i) if (i * 256 + tid < KN) rk[i] = *(const v8*)(kp + (i * 256 + tid) * 8);
+#pragma unroll
+        for (int i = 0; i < VP; ++i) rv[i] = *(const v8*)(vp + (i * 256 + tid) * 8);
+    };
+    auto lay = [&](int stage) {
+        T* ks = smem + stage * (KE + VE);
+        T* vs = ks + KE;
+#pragma unroll
+        for (int i = 0; i < KP; ++i) if (i * 256 + tid < KN) *(v8*)(ks + (i * 256 + tid) * 8) = rk[i];
+#pragma unroll
+        for (int i = 0; i < VP; ++i) *(v8*)(vs + (i * 256 + tid) * 8) = rv[i];
+    };
+    fetch(P0);
+    lay(0);
+    __syncthreads();
+    f32x16 s[2];
+    for (int p = P0; p < P1; ++p) {
+        const int stage = (p - P0) & 1;
+        if (p + 1 < P1) fetch(p + 1);
+        if (p >= p0 && p < p1) {
+            const T* ks = smem + stage * (KE + VE);
+            const T* vs = ks + KE;
+            v8 kf[2 * KS], vf[DB * 4];
+            a.load_k(ks, kf);
+            a.load_v(vs, vf);
+            const bool inside = all_valid && p * PAGE >= lo_max && p * PAGE + PAGE - 1 <= pos_min;
+            a.weights(kf, s, p * PAGE, lo, hi, scale2, bias2, !inside);
+            a.mix(vf, s);
+        }
+        if (p + 1 < P1) lay(stage ^ 1);
+        __syncthreads();
     }
     if (!valid) return;
     T* orow = out + (tok * H + h) * dv;
@@ -212,8 +258,17 @@ template <class T>
 __global__ void sigmoid_merge_kernel(const float* __restrict__ part, T* __restrict__ out, int S, int dv) {
     const int64_t bh = blockIdx.x;
     for (int d = threadIdx.x; d < dv; d += blockDim.x) {
+        const float* p = part + bh * S * dv + d;
         float acc = 0.f;
-        for (int s = 0; s < S; ++s) acc += part[(bh * S + s) * dv + d];
+        int s = 0;
+        for (; s + 8 <= S; s += 8) {               // eight loads in flight, added in ascending order
+            float v[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = p[(int64_t)(s + i) * dv];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc += v[i];
+        }
+        for (; s < S; ++s) acc += p[(int64_t)s * dv];
         out[bh * dv + d] = from_f32<T>(acc);
     }
 }
@@ -235,8 +290,16 @@ extern "C" int li_sigattn_prefill(const void* q, void* out, int dt, const void* 
     if (n_tiles <= 0) return LI_OK;
     CachePtrs c{k, v, page_stride, page_table, max_pages};
     dim3 grid(n_tiles, H), block(256);
-#define GO(T) sigmoid_prefill_kernel<T><<<grid, block, 0, stream>>>((const T*)q, (T*)out, c, tile_seq, tile_q0, seq_slot, \
-        seq_qstart, seq_qlen, seq_ctx, bias, H, G, dv, scale, window)
+    const size_t lds = (size_t)2 * (PAGE * KD + PAGE * DB * 32) * 2;
+#define GO(T)                                                                                                        \
+    do {                                                                                                             \
+        auto kfn = sigmoid_prefill_kernel<T>;                                                                        \
+        if (lds > 48 * 1024 &&                                                                                       \
+            hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)  \
+            return LI_HIP_ERROR;                                                                                     \
+        kfn<<<grid, block, lds, stream>>>((const T*)q, (T*)out, c, tile_seq, tile_q0, seq_slot, seq_qstart, seq_qlen,  \
+                                          seq_ctx, bias, H, G, dv, scale, window);                                   \
+    } while (0)
     if (dt == DT_F16) GO(f16); else if (dt == DT_BF16) GO(bf16); else return LI_BAD_ARG;
 #undef GO
     LI_CHECK_LAUNCH();
@@ -256,7 +319,7 @@ extern "C" int li_sigattn_decode(const void* q, void* out, int dt, const void* k
     do {                                                                                                             \
         sigmoid_decode_kernel<T><<<grid, block, 0, stream>>>((const T*)q, (T*)out, part, c, seq_slot, seq_ctx, bias, H, G, \
                                                              dv, scale, window);                                     \
-        if (splits > 1) sigmoid_merge_kernel<T><<<n_seqs * H, 64, 0, stream>>>(part, (T*)out, splits, dv);          \
+        if (splits > 1) sigmoid_merge_kernel<T><<<n_seqs * H, dv <= 64 ? 64 : (dv <= 128 ? 128 : 256), 0, stream>>>(part, (T*)out, splits, dv); \
     } while (0)
     if (dt == DT_F16) GO(f16); else if (dt == DT_BF16) GO(bf16); else return LI_BAD_ARG;
 #undef GO

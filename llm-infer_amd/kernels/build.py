@@ -213,8 +213,8 @@ def build_all(head_dims=(16, 32, 48, 64, 128), force=True, sigmoid_head_dims=((4
     sigmoid attention library for each pair of head sizes given."""
     core_library(force=force)
     mixers_library(force=force)
-    for kd, vd in sigmoid_head_dims:
-        _build_library(*_sigmoid_attention_args(kd, vd), force)
+    with ThreadPoolExecutor(max_workers=4) as pool:
+        list(pool.map(lambda p: _build_library(*_sigmoid_attention_args(*p), force), sigmoid_head_dims))
     with ThreadPoolExecutor(max_workers=4) as pool:
         list(pool.map(lambda hd: _build_library(f"libli_attn_hd{hd}.so", (ATTN_SOURCE,),
                                                 (f"-DHEAD_DIM={hd}",), force), head_dims))

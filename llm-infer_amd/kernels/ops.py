@@ -880,9 +880,10 @@ def cast(x: torch.Tensor, dtype) -> torch.Tensor:
     return out
 
 
-def token_shift(x, mu, state, pos, tok_slot, out_dtype) -> torch.Tensor:
+def token_shift(x, mu, state, pos, tok_slot, out_dtype, single: bool = False) -> torch.Tensor:
     """out_t = x_t + (x_{t-1} - x_t) * mu with the row before from this step or from ``state[slot]`` (zeros at
-    position 0); afterwards ``state[slot]`` holds each sequence's last row of this step."""
+    position 0); afterwards ``state[slot]`` holds each sequence's last row of this step.  ``single``: every
+    sequence brings exactly one row (a decode step), which one kernel then serves."""
     _dev(x, mu, state, pos, tok_slot)
     _f32_rows(x, "token_shift x")
     t, d = x.shape
@@ -892,7 +893,7 @@ def token_shift(x, mu, state, pos, tok_slot, out_dtype) -> torch.Tensor:
           "token_shift: int32 positions and slots for every token")
     out = torch.empty((t, d), dtype=out_dtype, device=x.device)
     _check(mixers().li_token_shift(_ptr(x), _ptr(mu), _ptr(state), _ptr(pos), _ptr(tok_slot), _ptr(out), DT[out_dtype],
-                                   t, d, _stream()), "token_shift")
+                                   t, d, int(bool(single)), _stream()), "token_shift")
     return out
 
 

@@ -40,7 +40,8 @@ class ShiftedMixer(Part):
         return [StateSpec((self.hidden_size,), "float32")] + cache_specs_of(self.inner)
 
     def _shift(self, x, ctx, views):
-        return ops.token_shift(x, self.mu, views[0].state, ctx.pos, ctx.tok_slot, self.dtype)
+        return ops.token_shift(x, self.mu, views[0].state, ctx.pos, ctx.tok_slot, self.dtype,
+                               single=ctx.n_tokens == ctx.n_seqs)
 
     def addends(self, x, ctx, views, owns_cache=True):
         if not owns_cache:
