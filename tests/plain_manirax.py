@@ -75,17 +75,19 @@ def rotate_half_layout(v, positions, base, dims, factor):
     return out
 
 
-def sigmoid_attention(q, k, v, scale, bias):
+def sigmoid_attention(q, k, v, scale, bias, window=None):
     """q [T, H, d], k [T, G, d], v [T, G, dv], bias [H].  Token t takes sum over j <= t of
-    sigmoid(q_t . k_j * scale + bias_h) v_j; query head h reads key/value head h // (H / G)."""
+    sigmoid(q_t . k_j * scale + bias_h) v_j; query head h reads key/value head h // (H / G).
+    ``window`` (not part of the design; the library's mixer offers it): only the last ``window`` keys, t included."""
     T, H, _ = q.shape
     G = k.shape[1]
     out = torch.zeros((T, H, v.shape[-1]), dtype=q.dtype)
     for h in range(H):
         g = h // (H // G)
         for t in range(T):
-            s = (k[:t + 1, g] @ q[t, h]) * scale + bias[h]
-            out[t, h] = torch.sigmoid(s) @ v[:t + 1, g]
+            lo = 0 if window is None else max(0, t - window + 1)
+            s = (k[lo:t + 1, g] @ q[t, h]) * scale + bias[h]
+            out[t, h] = torch.sigmoid(s) @ v[lo:t + 1, g]
     return out
 
 

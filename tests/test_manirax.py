@@ -191,3 +191,10 @@ def test_plain_model_is_causal_and_layered(name):
     other = copy.deepcopy(cfg)
     other["layers"][0]["mixer"]["right_scale"] += 0.5
     assert (P.forward(W, other, toks) - logits).abs().max() > 1e-3
+
+
+def test_chunk_lists_of_the_decay_attention():
+    from llm_infer_amd.kernels import ops
+    assert ops.DECAY_CHUNK == 32
+    seq, t0, first = ops.decay_chunk_lists([70, 1, 32, 33])
+    assert seq == [0, 0, 0, 1, 2, 3, 3] and t0 == [0, 32, 64, 0, 0, 0, 32] and first == [0, 3, 4, 5]

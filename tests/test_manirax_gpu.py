@@ -404,3 +404,54 @@ def test_trace_replay_in_three_schedules(lib, models, dtype, tmp_path):
         out = TU.run_trace(folder, dtype, steps, where, cfg["vocab"], 512, str(tmp_path / f"{dtype}{k}"))
         for (r, p), row in out.items():
             assert M.row_error(torch.from_numpy(row)[None], refs[r][p:p + 1]) < TOL[dtype], (k, r, p)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sigmoid_attention_window_edges(lib, dtype):
+    """The mixer's optional window (the design itself has none): a key exactly at the window's edge counts, the
+    one before it does not, in a prompt, in a portion that continues it and in decoding, with the keys that
+    decide made to stand out."""
+    from llm_infer_amd.cache import Cache
+    from llm_infer_amd.cache.specs import KVSpec
+    from llm_infer_amd.kernels import ops
+    dt = DT[dtype]
+    g = torch.Generator().manual_seed(9)
+    H, G, d, dv, T, W = 2, 1, 32, 32, 200, 70
+    k, v, q = torch.randn(T, G, d, generator=g), torch.randn(T, G, dv, generator=g), torch.randn(T, H, d, generator=g)
+    for t in (100, 150, 199, 69, 70):            # queries that look at the key just inside and just outside
+        q[t, 0] = k[max(0, t - W + 1), 0] * 5.0
+        q[t, 1] = k[max(0, t - W), 0] * 5.0
+    bias = torch.full((H,), -0.8 * d)
+    ref = P.sigmoid_attention(P.unit_rms(q.double(), 0.0), P.unit_rms(k.double(), 0.0), v.double(), 1.0, bias.double(), window=W)
+    assert (ref[150, 0] - v[81, 0].double()).abs().max() < 0.05 and ref[150, 1].abs().max() < 0.05
+    cache = Cache([KVSpec(G, d, W, dv)], 1024, 1024, dt, DEV)
+    slot = cache.alloc_slot()
+    got, at = [], 0
+    for n in [130, 40] + [1] * 30:               # a prompt, a portion, then token by token
+        cache.grow([slot], [at + n], filled=True)
+        ctx = ctx_for([at], [[0] * n])
+        rows = slice(at, at + n)
+        qkv = torch.cat([q[rows].reshape(n, -1), k[rows].reshape(n, -1), v[rows].reshape(n, -1)], 1).to(DEV)
+        kv = cache.view(0).as_tuple()
+        qd = ops.rope_norm_store(qkv, None, 0, False, 0.0, ctx.pos, ctx.tok_slot, kv, H, G, d, dv, d, d, dv, dt)
+        if dtype == "float32":
+            out = ops.sigmoid_attention(qd, kv, ctx.pos, ctx.tok_slot, bias.to(DEV), H, G, d, dv, dv, 1.0, W)
+        elif ctx.is_decode:
+            out = ops.sigmoid_attention_decode(qd, kv, ctx.seq_slot, ctx.seq_ctx, 1, bias.to(DEV), H, G, d, dv, dv, 1.0, W, 2)
+        else:
+            out = ops.sigmoid_attention_prefill(qd, kv, ops.prefill_meta(ctx), bias.to(DEV), H, G, d, dv, dv, 1.0, W)
+        got.append(out.cpu().double())
+        at += n
+        cache.trim_windows([slot])
+    assert at == T
+    assert (torch.cat(got) - ref).abs().max() < (1e-4 if dtype == "float32" else 3e-2)
+
+
+def test_float16_runs_the_same_kernels(lib, models):
+    folder, cfg, W = models["Q"]
+    eng = lib.load(folder, dtype="float16", max_tokens=1024)
+    toks = tokens(cfg, 100, 8)
+    ref = P.forward(W, cfg, toks)
+    s = eng.alloc_slot()
+    rows = [eng.step([s], [toks[:90]], [all_rows(90)]).cpu()] + [eng.step([s], [[t]], [[0]]).cpu() for t in toks[90:]]
+    assert M.row_error(torch.cat(rows), ref) < 1e-2
