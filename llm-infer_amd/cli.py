@@ -117,11 +117,11 @@ def run(cfg) -> int:
         config = llm_infer_amd.config_from_folder(cfg["model"])
     if cfg["context"]:
         raw = config.to_dict()
-        raw["max_position_embeddings"] = cfg["context"]
+        raw[config.context_key] = cfg["context"]         # each configuration class names its own key
         raw["eos_token_id"] = list(config.eos_token_ids) or None
         config = llm_infer_amd.config_from_dict(raw)
     tok = None if cfg["config"] else Tokenizer.from_model(
-        cfg["model"], config.bos_token_id, config.eos_token_ids[0] if config.eos_token_ids else None)
+        cfg["model"], getattr(config, "bos_token_id", None), config.eos_token_ids[0] if config.eos_token_ids else None)
     if cfg["prompt_file"]:
         try:
             with open(cfg["prompt_file"], encoding="utf-8") as f:
@@ -141,8 +141,8 @@ def run(cfg) -> int:
     if cfg["slots"] is not None and cfg["slots"] <= 0:
         raise RuntimeError("--slots must be positive")
     n_slots = min(cfg["slots"] or len(prompts), len(prompts)) or 1
-    each = sorted((-(-min(len(p) + cfg["max_tokens"], config.max_position_embeddings) // 64) * 64 for p in prompts),
-                  reverse=True)
+    bound = getattr(config, config.context_key) or (1 << 62)      # 0: the design sets no bound on positions
+    each = sorted((-(-min(len(p) + cfg["max_tokens"], bound) // 64) * 64 for p in prompts), reverse=True)
     need = sum(each[:n_slots])                       # the largest batch that can be live at once
     if cfg["random"]:
         engine = Engine.from_random(config, seed=cfg["seed_weights"], dtype=cfg["dtype"], max_tokens=need,
@@ -154,11 +154,8 @@ def run(cfg) -> int:
         if cfg["context"]:
             engine.max_positions = min(engine.max_positions, cfg["context"])
     print("Model load successful")
-    print(f"  Layers: {config.num_hidden_layers}")
-    print(f"  Dimensions: {config.hidden_size}")
-    print(f"  Heads: {config.num_attention_heads}")
-    print(f"  KV Heads: {config.num_key_value_heads}")
-    print(f"  Vocab size: {config.vocab_size}")
+    for label, value in config.summary():
+        print(f"  {label}: {value}")
     print(f"  Max seq len: {engine.max_positions}")
     print(f"  Device: {cfg['device']}")
     print()

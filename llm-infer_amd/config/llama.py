@@ -188,6 +188,14 @@ class LlamaConfig:
         if not self.rope_theta > 0 or not self.rms_norm_eps >= 0:
             raise ConfigError("rope_theta must be positive and rms_norm_eps non-negative")
 
+    context_key = "max_position_embeddings"       # the key (and field) that bounds a sequence's positions
+
+    def summary(self) -> list:
+        """(label, value) lines for the command line's report (tools/infer.cpp:248-255)."""
+        return [("Layers", self.num_hidden_layers), ("Dimensions", self.hidden_size),
+                ("Heads", self.num_attention_heads), ("KV Heads", self.num_key_value_heads),
+                ("Vocab size", self.vocab_size)]
+
     def to_dict(self) -> dict:
         """The config.json that reads back as this configuration."""
         out = {

@@ -97,6 +97,17 @@ class ManiraxConfig:
                 if int(_need(mlp, "ff", where + " mlp")) <= 0:
                     raise ConfigError(f"{where} mlp: ff must be positive")
 
+    context_key = "max_positions"                 # the optional key (and field) that bounds a sequence's positions
+
+    def summary(self) -> list:
+        """(label, value) lines for the command line's report."""
+        left = [layer["mixer"]["left"] for layer in self.layers]
+        right = [layer["mixer"]["right"] for layer in self.layers]
+        span = lambda xs: str(xs[0]) if len(set(xs)) == 1 else f"{min(xs)}..{max(xs)}"
+        return [("Layers", len(self.layers)), ("Dimensions", self.width),
+                ("Heads", span([int(l["heads"]) for l in left]) + " sigmoid + " + span([int(r["heads"]) for r in right]) + " linear"),
+                ("KV Heads", span([int(l["kv_heads"]) for l in left])), ("Vocab size", self.vocab)]
+
     def to_dict(self) -> dict:
         """The config.json that reads back as this configuration."""
         out = {"architecture": self.architecture, "layers": copy.deepcopy(list(self.layers)),

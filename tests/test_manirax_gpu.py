@@ -2,7 +2,10 @@
 into portions, decoding token by token, batches of unequal requests, slots and pages used again, keys far
 away and at page borders, long decoding, and greedy generation through the library's entry point."""
 import copy
+import json
 import os
+import subprocess
+import sys
 
 import pytest
 import torch
@@ -455,3 +458,25 @@ def test_float16_runs_the_same_kernels(lib, models):
     s = eng.alloc_slot()
     rows = [eng.step([s], [toks[:90]], [all_rows(90)]).cpu()] + [eng.step([s], [[t]], [[0]]).cpu() for t in toks[90:]]
     assert M.row_error(torch.cat(rows), ref) < 1e-2
+
+
+def test_command_line_and_model_info(lib, models):
+    folder, cfg, W = models["P"]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    prompts = [tokens(cfg, 9, 51), tokens(cfg, 2, 52)]
+    cmd = [sys.executable, os.path.join(root, "bin", "infer"), folder, "-n", "6", "-t", "0", "--dtype", "float32", "-T", "64"]
+    for p in prompts:
+        cmd += ["--tokens", ",".join(map(str, p))]
+    res = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0, res.stderr
+    got = [json.loads(line.split("tokens: ", 1)[1]) for line in res.stdout.splitlines() if " tokens: [" in line]
+    for p, new in zip(prompts, got):
+        toks = list(p)
+        for t in new:
+            assert t == int(P.forward(W, cfg, toks)[-1].argmax())
+            toks.append(t)
+    for word in ("Layers: 2", "Dimensions: 72", "Heads: 2..6 sigmoid + 2..3 linear", "Vocab size: 131", "Max seq len: 64"):
+        assert word in res.stdout, res.stdout
+    info = subprocess.run([sys.executable, os.path.join(root, "bin", "model_info"), folder], capture_output=True, text=True,
+                          timeout=300)
+    assert info.returncode == 0 and "Architecture: Manirax" in info.stdout and "The tensors fit the model." in info.stdout
