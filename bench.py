@@ -151,11 +151,11 @@ def compare_configs(design: str, size: dict, layers: int, context: int) -> dict:
     # the attention of the same heads beside a linear attention of half as many heads with states of hd x hd
     layer = {"type": "parallel", "mlp": {"kind": "dense", "ff": size["ff"]},
              "mixer": {"left": {"heads": H, "kv_heads": G, "dim": hd, "vdim": hd, "scale": hd ** -0.5,
-                                "rot": {"base": 500000.0, "dims": hd // 2, "scaling": {"factor": 4.0}}},
+                                "rot": {"base": 500000.0, "dims": hd // 2, "scaling": {"factor": 2.0}}},
                        "right": {"heads": H // 2, "dim": hd, "vdim": hd,
                                  "decay": [1.0 - 2.0 ** -(3 + 5 * i / max(1, H // 2 - 1)) for i in range(H // 2)]},
-                       "left_scale": 0.8, "right_scale": 1.1}}
-    other = {"architecture": "Manirax", "layers": [layer] * layers, "norm": {"eps": 1e-5}, "postln_alpha": 2.5,
+                       "left_scale": 1.0, "right_scale": 1.0}}
+    other = {"architecture": "Manirax", "layers": [layer] * layers, "norm": {"eps": 1e-5}, "postln_alpha": 2.0,
              "vocab": size["vocab"], "width": w, "max_positions": context}
     return {"llama": llama, design: other}
 

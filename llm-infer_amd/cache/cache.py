@@ -21,6 +21,7 @@ caller passes (src/model/model.cpp:66-68).
 """
 from __future__ import annotations
 
+import math
 from dataclasses import dataclass
 
 import numpy as np
@@ -32,6 +33,7 @@ from .specs import KVSpec, StateSpec
 
 PAGE = 64
 NULL_PAGE = 0
+STATE_BUDGET = 8 << 30       # bytes that the state groups may take when the caller does not say how many slots
 
 
 def _round_up(a: int, b: int) -> int:
@@ -185,7 +187,15 @@ class Cache:
             raise CacheError("kv_round: float16 or bfloat16, for a float32 cache (a 16-bit cache rounds to its own type)")
         self.max_positions = max_positions
         self.n_pages = max(1, (max_tokens + PAGE - 1) // PAGE) + 1          # page 0 is never handed out
-        self.n_slots = n_slots or max(1, min(self.n_pages - 1, 4096))
+        if n_slots is None:
+            # as many slots as there are pages (a sequence holds at least one), unless the fixed-size states of
+            # that many sequences would outgrow STATE_BUDGET: a mixer's state may be a megabyte a layer
+            n_slots = max(1, min(self.n_pages - 1, 4096))
+            per_slot = sum(math.prod(s.shape) * torch.empty((), dtype=getattr(torch, s.dtype)).element_size()
+                           for s in specs if isinstance(s, StateSpec))
+            if per_slot:
+                n_slots = max(1, min(n_slots, max(16, STATE_BUDGET // per_slot)))
+        self.n_slots = n_slots
         self.device, self.dtype = device, dtype
         self.slots = SlotAllocator(self.n_slots)
         self.scratch_slot = self.n_slots          # behind the last slot in every per-slot table; never handed out

@@ -42,13 +42,13 @@ TINY_P = config(72, 131, [
 TINY_Q = config(64, 97, [
     layer(left(4, 4, 32, 48, rot={"base": 100.0, "dims": 32}), right(1, 16, 16, [1.0]), 1.0, 1.0, 48),
     layer(left(3, 1, 48, 16), right(4, 16, 8, [0.3, 0.6, 0.9, 0.97]), 0.5, 2.0, 136),
-    layer(left(1, 1, 64, 64, rot={"base": 1e6, "dims": 2, "scaling": {"factor": 8.0}}),
+    layer(left(1, 1, 64, 64, rot={"base": 2e5, "dims": 2, "scaling": {"factor": 8.0}}),
           right(2, 32, 32, [0.999, 0.5]), 1.2, 0.8, 64),
 ], eps=1e-4, alpha=1.0)
 
 # wider heads (the sizes of real layers, few of them): 128-wide keys and values, a linear state of 128 x 128
 TINY_R = config(256, 211, [
-    layer(left(4, 2, 128, 128, rot={"base": 10000.0, "dims": 64, "scaling": {"factor": 4.0}}),
+    layer(left(4, 2, 128, 128, rot={"base": 10000.0, "dims": 64, "scaling": {"factor": 3.0}}),
           right(2, 128, 128, [0.9, 0.99]), 0.9, 1.1, 384),
 ], eps=1e-5, alpha=2.0)
 

@@ -198,3 +198,16 @@ def test_chunk_lists_of_the_decay_attention():
     assert ops.DECAY_CHUNK == 32
     seq, t0, first = ops.decay_chunk_lists([70, 1, 32, 33])
     assert seq == [0, 0, 0, 1, 2, 3, 3] and t0 == [0, 32, 64, 0, 0, 0, 32] and first == [0, 3, 4, 5]
+
+
+def test_default_slots_are_capped_by_the_states_memory():
+    from llm_infer_amd.cache import Cache
+    from llm_infer_amd.cache.cache import STATE_BUDGET
+    from llm_infer_amd.cache.specs import KVSpec, StateSpec
+    big = StateSpec((16, 128, 128))                         # a megabyte a layer and sequence
+    cache = Cache([KVSpec(2, 64), big, big], 1 << 20, 4096, torch.bfloat16, None)
+    assert cache.n_slots == STATE_BUDGET // (2 * 16 * 128 * 128 * 4) == 4096
+    cache = Cache([KVSpec(2, 64)] + [big] * 64, 1 << 20, 4096, torch.bfloat16, None)
+    assert cache.n_slots == STATE_BUDGET // (64 * 16 * 128 * 128 * 4) == 128
+    assert Cache([KVSpec(2, 64)] + [big] * 64, 1 << 20, 4096, torch.bfloat16, None, n_slots=300).n_slots == 300
+    assert Cache([KVSpec(2, 64)], 640, 4096, torch.bfloat16, None).n_slots == 10
