@@ -232,7 +232,9 @@ extern "C" int li_token_shift(const float* x, const float* mu, float* state, con
                               void* out, int out_dt, int n_tokens, int d, int single, hipStream_t stream) {
     if (n_tokens <= 0) return LI_OK;
     if (d <= 0) return LI_BAD_ARG;
-    dim3 grid(n_tokens), block(d >= 1024 ? 256 : 64);
+    // a few rows (a decode step): as many threads a row as it has elements to four, so that a thread's loads are few
+    const int wide = min(1024, (d / 4 + 63) / 64 * 64);
+    dim3 grid(n_tokens), block(n_tokens < 256 && wide > 64 ? wide : (d >= 1024 ? 256 : 64));
     if (out_dt == DT_F32) token_shift_kernel<float><<<grid, block, 0, stream>>>(x, mu, state, pos, tok_slot, (float*)out, d, single);
     else if (out_dt == DT_F16) token_shift_kernel<f16><<<grid, block, 0, stream>>>(x, mu, state, pos, tok_slot, (f16*)out, d, single);
     else if (out_dt == DT_BF16) token_shift_kernel<bf16><<<grid, block, 0, stream>>>(x, mu, state, pos, tok_slot, (bf16*)out, d, single);
@@ -748,7 +750,8 @@ extern "C" int li_gated_rmsnorm(const float* o, const float* w, const float* gat
                                 int out_dt, int n_rows, int n, float eps, hipStream_t stream) {
     if (n_rows <= 0) return LI_OK;
     if (n <= 0 || gate_stride < n) return LI_BAD_ARG;
-    dim3 grid(n_rows), block(n >= 1024 ? 256 : 64);
+    const int wide = min(1024, (n / 4 + 63) / 64 * 64);
+    dim3 grid(n_rows), block(n_rows < 256 && wide > 64 ? wide : (n >= 1024 ? 256 : 64));
     if (out_dt == DT_F32) gated_rmsnorm_kernel<float><<<grid, block, 0, stream>>>(o, w, gate, gate_stride, (float*)out, n, eps);
     else if (out_dt == DT_F16) gated_rmsnorm_kernel<f16><<<grid, block, 0, stream>>>(o, w, gate, gate_stride, (f16*)out, n, eps);
     else if (out_dt == DT_BF16) gated_rmsnorm_kernel<bf16><<<grid, block, 0, stream>>>(o, w, gate, gate_stride, (bf16*)out, n, eps);

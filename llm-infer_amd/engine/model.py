@@ -104,6 +104,14 @@ class DecoderModel(Part):
             part.bind({local: tensors[name] for local, name in names})
         if getattr(self.head, "tied", False):
             self.head.tie(self.embedding.weight)
+        # parts that arrange something across their children once all have their tensors (a product shared by
+        # mixers that read the same rows)
+        stack = list(self.children())
+        while stack:
+            part = stack.pop()
+            if hasattr(part, "finish_bind"):
+                part.finish_bind()
+            stack += list(part.children())
 
     # -- cache -------------------------------------------------------------
     def cache_specs(self) -> list:

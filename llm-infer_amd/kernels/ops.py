@@ -898,16 +898,17 @@ def token_shift(x, mu, state, pos, tok_slot, out_dtype, single: bool = False) ->
 
 
 def rope_norm_store(qkv, inv_freq, rotary_dim, half_pairing, unit_eps, pos, tok_slot, kv, n_heads, n_kv_heads,
-                    head_dim, v_head_dim, q_dim, k_dim, v_dim, out_dtype) -> torch.Tensor:
+                    head_dim, v_head_dim, q_dim, k_dim, v_dim, out_dtype, col0: int = 0) -> torch.Tensor:
     """q and k of a step rotated by position (half or adjacent pairing), then, with ``unit_eps`` not None,
     divided by their root mean square per head; k and v written into the pages (``kv`` = (k_pages, v_pages,
     page_stride, page_table); head sizes ``k_dim`` and ``v_dim`` in the pages, zeros beyond the true ones).
+    ``col0``: the column of ``qkv`` at which q begins (a product shared with other mixers).
     Returns q [T, H, q_dim]."""
     k_pages, v_pages, page_stride, page_table = kv
     _dev(qkv, inv_freq, pos, tok_slot, k_pages, v_pages, page_table)
     _f32_rows(qkv, "rope_norm_store qkv")
     t = qkv.shape[0]
-    _need(qkv.shape[1] >= (n_heads + n_kv_heads) * head_dim + n_kv_heads * v_head_dim, "qkv row too short")
+    _need(col0 >= 0 and qkv.shape[1] >= col0 + (n_heads + n_kv_heads) * head_dim + n_kv_heads * v_head_dim, "qkv row too short")
     _need(pos.dtype == torch.int32 and tok_slot.dtype == torch.int32 and pos.numel() >= t and tok_slot.numel() >= t,
           "int32 positions and slots for every token")
     _need(max(head_dim, q_dim, k_dim, v_dim) <= 256 and q_dim >= head_dim and k_dim >= head_dim and v_dim >= v_head_dim
@@ -919,7 +920,7 @@ def rope_norm_store(qkv, inv_freq, rotary_dim, half_pairing, unit_eps, pos, tok_
     _need(page_table.dtype == torch.int32 and page_table.dim() == 2, "page_table: int32 [slots, pages]")
     q = torch.empty((t, n_heads, q_dim), dtype=out_dtype, device=qkv.device)
     _check(mixers().li_rope_norm_store(
-        _ptr(qkv), qkv.shape[1], _ptr(inv_freq), rotary_dim, int(half_pairing),
+        c_void_p(qkv.data_ptr() + 4 * col0), qkv.shape[1], _ptr(inv_freq), rotary_dim, int(half_pairing),
         c_float(-1.0 if unit_eps is None else unit_eps), _ptr(pos), _ptr(tok_slot), _ptr(k_pages), _ptr(v_pages),
         c_int64(page_stride), _ptr(page_table), page_table.shape[1], _ptr(q), DT[out_dtype], t, n_heads, n_kv_heads,
         head_dim, v_head_dim, q_dim, k_dim, v_dim, _stream()), "rope_norm_store")

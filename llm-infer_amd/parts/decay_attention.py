@@ -51,20 +51,25 @@ class DecayLinearAttention(Part):
     def cache_spec(self):
         return StateSpec((self.n_heads, self.head_dim, self.v_head_dim), "float32")
 
-    def addends(self, h, ctx, view, owns_cache=True):
+    def in_rows(self) -> int:
+        return 2 * self.n_heads * (self.head_dim + self.v_head_dim)
+
+    def addends(self, h, ctx, view, owns_cache=True, proj=None, col0=0):
+        """``proj`` (float32 [T, n]) with this mixer's q, k, v, g from column ``col0`` on: the product is not run here."""
         if not owns_cache:
             raise ValueError("decay attention keeps a state of its own in every run")
         H, d, dv = self.n_heads, self.head_dim, self.v_head_dim
-        proj = ops.linear(h, self.w_in, out_dtype=torch.float32)
+        if proj is None:
+            proj, col0 = ops.linear(h, self.w_in, out_dtype=torch.float32), 0
         # a 16-bit model: prompts run 32 tokens at a time on the matrix cores, decoding token by token on the same
         # 16-bit values of q, k and v; a float32 model runs token by token throughout
         sixteen = self.dtype != torch.float32
         chunked = sixteen and not ctx.is_decode
-        o = ops.decay_attention(proj, 0, H * d, 2 * H * d, view.state, self.decay, ctx.seq_slot,
+        o = ops.decay_attention(proj, col0, col0 + H * d, col0 + 2 * H * d, view.state, self.decay, ctx.seq_slot,
                                 getattr(ctx, "seq_qstart", None), getattr(ctx, "seq_qlen", None), ctx.n_seqs, H, d, dv,
                                 round_to=self.dtype if sixteen else None, chunked=chunked,
                                 chunks=ops.decay_chunks(ctx) if chunked else None)
-        a = ops.gated_rmsnorm(o, self.norm, proj, 2 * H * d + H * dv, self.norm_eps, self.dtype)
+        a = ops.gated_rmsnorm(o, self.norm, proj, col0 + 2 * H * d + H * dv, self.norm_eps, self.dtype)
         return [(ops.linear(a, self.wo, out_dtype=torch.float32), 1.0)]
 
     def forward(self, h, ctx, view, residual, owns_cache=True):

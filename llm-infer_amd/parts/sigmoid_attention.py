@@ -40,7 +40,7 @@ class SigmoidAttention(Part):
         self.head_bias = bool(head_bias)
         self.names = {**_NAMES, **(names or {})}
         self.prefix, self.dtype, self.device = prefix, dtype, device
-        self.wqkv = self.wo = self.bias = None
+        self.w_in = self.wo = self.bias = None
 
     def params(self):
         H, G, d, dv, w, n = self.n_heads, self.n_kv_heads, self.head_dim, self.v_head_dim, self.hidden_size, self.names
@@ -52,7 +52,9 @@ class SigmoidAttention(Part):
 
     def bind(self, tensors):
         n = self.names
-        self.wqkv = ops.prepare_weight(torch.cat([tensors[n["q"]], tensors[n["k"]], tensors[n["v"]]], 0).contiguous())
+        # ``w_in``: the stacked input matrix [Wq; Wk; Wv]; a mixer that runs this one beside others on the same rows
+        # may take it into a product of its own (``ParallelMixers``) and hand over the columns instead
+        self.w_in = ops.prepare_weight(torch.cat([tensors[n["q"]], tensors[n["k"]], tensors[n["v"]]], 0).contiguous())
         self.wo = ops.prepare_weight(tensors[n["o"]])
         self.bias = tensors[n["bias"]] if self.head_bias else None
 
@@ -66,15 +68,20 @@ class SigmoidAttention(Part):
             return None, 0, False
         return p.inv_freq, rot, getattr(p, "pairing", "adjacent") == "half"
 
-    def addends(self, h, ctx, view, owns_cache=True):
+    def in_rows(self) -> int:
+        return (self.n_heads + self.n_kv_heads) * self.head_dim + self.n_kv_heads * self.v_head_dim
+
+    def addends(self, h, ctx, view, owns_cache=True, proj=None, col0=0):
+        """``proj`` (float32 [T, n]) with this mixer's q, k, v from column ``col0`` on: the product is not run here."""
         if not owns_cache:
             raise ValueError("sigmoid attention writes its own keys and values in every run")
         H, G, d, dv = self.n_heads, self.n_kv_heads, self.head_dim, self.v_head_dim
-        qkv = ops.linear(h, self.wqkv, out_dtype=torch.float32)
+        if proj is None:
+            proj, col0 = ops.linear(h, self.w_in, out_dtype=torch.float32), 0
         inv_freq, rot, half = self._rotation()
         kv = view.as_tuple()
-        q = ops.rope_norm_store(qkv, inv_freq, rot, half, self.unit_norm_eps, ctx.pos, ctx.tok_slot, kv, H, G, d, dv,
-                                self.k_dim, self.k_dim, self.v_dim, self.dtype)
+        q = ops.rope_norm_store(proj, inv_freq, rot, half, self.unit_norm_eps, ctx.pos, ctx.tok_slot, kv, H, G, d, dv,
+                                self.k_dim, self.k_dim, self.v_dim, self.dtype, col0=col0)
         if self.dtype == torch.float32:
             a = ops.sigmoid_attention(q, kv, ctx.pos, ctx.tok_slot, self.bias, H, G, self.k_dim, dv, self.v_dim,
                                       self.scale, self.window)
