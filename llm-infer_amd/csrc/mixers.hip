@@ -123,12 +123,85 @@ __global__ __launch_bounds__(1024) void add_layernorm_reg_kernel(float* __restri
     }
 }
 
+// The same with 16-byte loads: N4 pieces of four elements a thread (d a multiple of 4, 16-byte aligned rows).
+template <class TC, int N4>
+__global__ __launch_bounds__(1024) void add_layernorm_vec_kernel(float* __restrict__ x, float alpha,
+                                                                 const float* __restrict__ y1, float s1,
+                                                                 const float* __restrict__ y2, float s2,
+                                                                 const float* __restrict__ w, float eps,
+                                                                 TC* __restrict__ copy, int d) {
+    struct alignas(4 * sizeof(TC)) Out4 { TC v[4]; };
+    __shared__ float scratch[16];
+    const int64_t base = (int64_t)blockIdx.x * d;
+    const int n4 = d >> 2;
+    f32x4* x4 = (f32x4*)(x + base);
+    const f32x4 *a4 = (const f32x4*)(y1 + base), *b4 = y2 ? (const f32x4*)(y2 + base) : nullptr, *w4 = (const f32x4*)w;
+    f32x4 v[N4];
+    float s = 0.f;
+#pragma unroll
+    for (int u = 0; u < N4; ++u) {
+        const int i = threadIdx.x + u * blockDim.x;
+        v[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (i < n4) {
+            const f32x4 xv = x4[i], av = a4[i];
+            f32x4 bv = {0.f, 0.f, 0.f, 0.f};
+            if (b4) bv = b4[i];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                float y = s1 * av[q];
+                if (b4) y += s2 * bv[q];
+                v[u][q] = alpha * xv[q] + y;
+                s += v[u][q];
+            }
+        }
+    }
+    const float mean = block_sum(s, scratch) / (float)d;
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < N4; ++u) {
+        const int i = threadIdx.x + u * blockDim.x;
+        if (i < n4) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) { v[u][q] -= mean; ss += v[u][q] * v[u][q]; }
+        }
+    }
+    const float sd = sqrtf(block_sum(ss, scratch) / (float)d + eps);
+#pragma unroll
+    for (int u = 0; u < N4; ++u) {
+        const int i = threadIdx.x + u * blockDim.x;
+        if (i < n4) {
+            const f32x4 wv = w4[i];
+            f32x4 r;
+            Out4 c4;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) { r[q] = v[u][q] / sd * wv[q]; c4.v[q] = from_f32<TC>(r[q]); }
+            x4[i] = r;
+            if (copy) ((Out4*)(copy + base))[i] = c4;
+        }
+    }
+}
+
 extern "C" int li_add_layernorm(float* x, float alpha, const float* y1, float s1, const float* y2, float s2,
                                 const float* w, float eps, void* copy, int copy_dt, int n_rows, int d,
                                 hipStream_t stream) {
     if (n_rows <= 0) return LI_OK;
     if (d <= 0 || !y1) return LI_BAD_ARG;
     dim3 grid(n_rows), block(d >= 2048 ? 512 : (d >= 256 ? 256 : 64));
+    const bool aligned = d % 4 == 0 && !(((uintptr_t)x | (uintptr_t)y1 | (uintptr_t)y2 | (uintptr_t)w | (uintptr_t)copy) & 15);
+    if (aligned && d <= 32 * 1024) {
+        const int n4 = d / 4, per = n4 <= 512 ? 1 : (n4 <= 1024 ? 2 : (n4 <= 4096 ? 4 : 8));
+        dim3 vb(((n4 + per - 1) / per + 63) / 64 * 64);
+#define GO1(TC, N) add_layernorm_vec_kernel<TC, N><<<grid, vb, 0, stream>>>(x, alpha, y1, s1, y2, s2, w, eps, (TC*)copy, d)
+#define GO(TC) do { if (per == 1) GO1(TC, 1); else if (per == 2) GO1(TC, 2); else if (per == 4) GO1(TC, 4); else GO1(TC, 8); } while (0)
+        if (!copy || copy_dt == DT_F32) GO(float);
+        else if (copy_dt == DT_F16) GO(f16);
+        else if (copy_dt == DT_BF16) GO(bf16);
+        else return LI_BAD_ARG;
+#undef GO
+#undef GO1
+        LI_CHECK_LAUNCH();
+        return LI_OK;
+    }
     if (d <= 8 * 1024) {
         const int per = d <= 4096 ? 4 : 8;
         dim3 rb(((d + per - 1) / per + 63) / 64 * 64);
@@ -251,7 +324,7 @@ extern "C" int li_token_shift(const float* x, const float* mu, float* state, con
 //   qkv [T, row_stride] float32: H query heads of d, then G key heads of d, then G value heads of dv
 // q and k: among the first `rot` dimensions of a head, dimension i is paired with i + rot/2 (half layout)
 // or 2j with 2j+1 (adjacent), and the pair (u, v) becomes (u cos a - v sin a, v cos a + u sin a) with
-// a = position * inv_freq[pair]; then, if unit_eps >= 0, the head is divided by sqrt(mean square + unit_eps).
+// a = position * inv_freq[pair] (or its cosine and sine from the step's table `cos_sin`, if given); then, if unit_eps >= 0, the head is divided by sqrt(mean square + unit_eps).
 // q goes to q_out [T, H, dq] (dq >= d, zeros beyond d), k and v into the token's page in the layout of
 // common.h with head sizes dk (>= d, a multiple of 16) and dvp (>= dv, a multiple of 16); what lies beyond
 // d and dv is written as zeros, up to the size the page holds.
@@ -259,9 +332,10 @@ extern "C" int li_token_shift(const float* x, const float* mu, float* state, con
 // ---------------------------------------------------------------------------
 template <class T>
 __global__ __launch_bounds__(256) void rope_norm_store_kernel(
-    const float* __restrict__ qkv, int row_stride, const float* __restrict__ inv_freq, int rot, int half_pairing,
-    float unit_eps, const int* __restrict__ pos, const int* __restrict__ tok_slot, Pages c, T* __restrict__ q_out,
-    int H, int G, int d, int dv, int dq, int dk, int dvp) {
+    const float* __restrict__ qkv, int row_stride, const float* __restrict__ inv_freq,
+    const float* __restrict__ cos_sin, int rot, int half_pairing, float unit_eps, const int* __restrict__ pos,
+    const int* __restrict__ tok_slot, Pages c, T* __restrict__ q_out, int H, int G, int d, int dv, int dq, int dk,
+    int dvp) {
     const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
     const int p = pos[t];
     const float* row = qkv + (int64_t)t * row_stride;
@@ -285,7 +359,12 @@ __global__ __launch_bounds__(256) void rope_norm_store_kernel(
                         if (half_pairing) { low = i < half; pair = low ? i : i - half; other = low ? i + half : i - half; }
                         else { low = !(i & 1); pair = i >> 1; other = i ^ 1; }
                         float sn, cs;
-                        sincosf((float)p * inv_freq[pair], &sn, &cs);
+                        if (cos_sin) {           // the step's table [T, rot / 2, 2]: the same two numbers, computed once
+                            cs = cos_sin[2 * ((int64_t)t * half + pair)];
+                            sn = cos_sin[2 * ((int64_t)t * half + pair) + 1];
+                        } else {
+                            sincosf((float)p * inv_freq[pair], &sn, &cs);
+                        }
                         const float o = src[other];
                         v = low ? v * cs - o * sn : v * cs + o * sn;
                     }
@@ -317,8 +396,8 @@ __global__ __launch_bounds__(256) void rope_norm_store_kernel(
     }
 }
 
-extern "C" int li_rope_norm_store(const float* qkv, int row_stride, const float* inv_freq, int rot, int half_pairing,
-                                  float unit_eps, const int* pos, const int* tok_slot, const void* k_pages,
+extern "C" int li_rope_norm_store(const float* qkv, int row_stride, const float* inv_freq, const float* cos_sin, int rot,
+                                  int half_pairing, float unit_eps, const int* pos, const int* tok_slot, const void* k_pages,
                                   const void* v_pages, int64_t page_stride, const int* page_table, int max_pages,
                                   void* q_out, int dt, int n_tokens, int H, int G, int d, int dv, int dq, int dk,
                                   int dvp, hipStream_t stream) {
@@ -329,7 +408,7 @@ extern "C" int li_rope_norm_store(const float* qkv, int row_stride, const float*
     Pages c{k_pages, v_pages, page_stride, page_table, max_pages};
     // few tokens: the heads spread over the grid as well
     dim3 grid(n_tokens, n_tokens >= 512 ? 1 : (H + 2 * G + 3) / 4), block(256);
-#define GO(T) rope_norm_store_kernel<T><<<grid, block, 0, stream>>>(qkv, row_stride, inv_freq, rot, half_pairing, \
+#define GO(T) rope_norm_store_kernel<T><<<grid, block, 0, stream>>>(qkv, row_stride, inv_freq, cos_sin, rot, half_pairing, \
         unit_eps, pos, tok_slot, c, (T*)q_out, H, G, d, dv, dq, dk, dvp)
     if (dt == DT_F32) GO(float); else if (dt == DT_F16) GO(f16); else if (dt == DT_BF16) GO(bf16); else return LI_BAD_ARG;
 #undef GO
@@ -814,11 +893,64 @@ __global__ void polynorm_reg_kernel(const float* __restrict__ z, const float* __
     }
 }
 
+// The same with 16-byte loads: N4 pieces of four elements a thread (n a multiple of 4, 16-byte aligned rows).
+template <class TO, int N4>
+__global__ __launch_bounds__(1024) void polynorm_vec_kernel(const float* __restrict__ z, const float* __restrict__ coef,
+                                                            TO* __restrict__ out, int n, float eps) {
+    struct alignas(4 * sizeof(TO)) Out4 { TO v[4]; };
+    __shared__ float scratch[16];
+    const int64_t base = (int64_t)blockIdx.x * n;
+    const int n4 = n >> 2;
+    const f32x4* z4 = (const f32x4*)(z + base);
+    f32x4 v[N4];
+    float s1 = 0.f, s2 = 0.f, s3 = 0.f;
+#pragma unroll
+    for (int u = 0; u < N4; ++u) {
+        const int i = threadIdx.x + u * blockDim.x;
+        v[u] = i < n4 ? z4[i] : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const float v2 = v[u][q] * v[u][q], v3 = v2 * v[u][q];
+            s1 += v2; s2 += v2 * v2; s3 += v3 * v3;
+        }
+    }
+    const float r1 = sqrtf(block_sum(s1, scratch) / (float)n + eps);
+    const float r2 = sqrtf(block_sum(s2, scratch) / (float)n + eps);
+    const float r3 = sqrtf(block_sum(s3, scratch) / (float)n + eps);
+    // a / r1, b / r2, c / r3 once a row: an element then costs three multiply-adds and no division
+    const float a1 = coef[0] / r1, b2 = coef[1] / r2, c3 = coef[2] / r3, e = coef[3];
+#pragma unroll
+    for (int u = 0; u < N4; ++u) {
+        const int i = threadIdx.x + u * blockDim.x;
+        if (i < n4) {
+            Out4 o4;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const float x = v[u][q], v2 = x * x, v3 = v2 * x;
+                o4.v[q] = from_f32<TO>(a1 * x + b2 * v2 + c3 * v3 + e);
+            }
+            ((Out4*)(out + base))[i] = o4;
+        }
+    }
+}
+
 extern "C" int li_polynorm(const float* z, const float* coef, void* out, int out_dt, int n_rows, int n, float eps,
                            hipStream_t stream) {
     if (n_rows <= 0) return LI_OK;
     if (n <= 0) return LI_BAD_ARG;
     dim3 grid(n_rows), block(n >= 2048 ? 512 : (n >= 256 ? 256 : 64));
+    if (n % 4 == 0 && n <= 32 * 1024 && !(((uintptr_t)z | (uintptr_t)out) & 15)) {
+        const int n4 = n / 4, per = n4 <= 512 ? 1 : (n4 <= 1024 ? 2 : (n4 <= 4096 ? 4 : 8));
+        dim3 vb(((n4 + per - 1) / per + 63) / 64 * 64);
+#define GO1(TO, N) polynorm_vec_kernel<TO, N><<<grid, vb, 0, stream>>>(z, coef, (TO*)out, n, eps)
+#define GO(TO) do { if (per == 1) GO1(TO, 1); else if (per == 2) GO1(TO, 2); else if (per == 4) GO1(TO, 4); else GO1(TO, 8); } while (0)
+        if (out_dt == DT_F32) GO(float); else if (out_dt == DT_F16) GO(f16); else if (out_dt == DT_BF16) GO(bf16);
+        else return LI_BAD_ARG;
+#undef GO
+#undef GO1
+        LI_CHECK_LAUNCH();
+        return LI_OK;
+    }
     if (n <= 16 * 1024) {
         dim3 rb(n <= 1024 ? 64 : (n <= 4096 ? 256 : (n <= 8192 ? 512 : 1024)));
         if (out_dt == DT_F32) polynorm_reg_kernel<float><<<grid, rb, 0, stream>>>(z, coef, (float*)out, n, eps);

@@ -898,11 +898,12 @@ def token_shift(x, mu, state, pos, tok_slot, out_dtype, single: bool = False) ->
 
 
 def rope_norm_store(qkv, inv_freq, rotary_dim, half_pairing, unit_eps, pos, tok_slot, kv, n_heads, n_kv_heads,
-                    head_dim, v_head_dim, q_dim, k_dim, v_dim, out_dtype, col0: int = 0) -> torch.Tensor:
+                    head_dim, v_head_dim, q_dim, k_dim, v_dim, out_dtype, col0: int = 0, cos_sin=None) -> torch.Tensor:
     """q and k of a step rotated by position (half or adjacent pairing), then, with ``unit_eps`` not None,
     divided by their root mean square per head; k and v written into the pages (``kv`` = (k_pages, v_pages,
     page_stride, page_table); head sizes ``k_dim`` and ``v_dim`` in the pages, zeros beyond the true ones).
-    ``col0``: the column of ``qkv`` at which q begins (a product shared with other mixers).
+    ``col0``: the column of ``qkv`` at which q begins (a product shared with other mixers).  ``cos_sin``: the
+    step's table of angles (``rope_table`` of the same frequencies and positions), read instead of computed.
     Returns q [T, H, q_dim]."""
     k_pages, v_pages, page_stride, page_table = kv
     _dev(qkv, inv_freq, pos, tok_slot, k_pages, v_pages, page_table)
@@ -918,9 +919,15 @@ def rope_norm_store(qkv, inv_freq, rotary_dim, half_pairing, unit_eps, pos, tok_
               "inv_freq: float32 [rotary_dim / 2]")
     _need(k_pages.dtype == out_dtype and v_pages.dtype == out_dtype, "cache dtype differs from q dtype")
     _need(page_table.dtype == torch.int32 and page_table.dim() == 2, "page_table: int32 [slots, pages]")
+    if cos_sin is not None and rotary_dim > 0:
+        _dev(cos_sin)
+        _need(cos_sin.dtype == torch.float32 and cos_sin.dim() == 3 and cos_sin.shape[0] >= t and
+              cos_sin.shape[1:] == (rotary_dim // 2, 2), "cos_sin: float32 [T, rotary_dim / 2, 2]")
+    else:
+        cos_sin = None
     q = torch.empty((t, n_heads, q_dim), dtype=out_dtype, device=qkv.device)
     _check(mixers().li_rope_norm_store(
-        c_void_p(qkv.data_ptr() + 4 * col0), qkv.shape[1], _ptr(inv_freq), rotary_dim, int(half_pairing),
+        c_void_p(qkv.data_ptr() + 4 * col0), qkv.shape[1], _ptr(inv_freq), _ptr(cos_sin), rotary_dim, int(half_pairing),
         c_float(-1.0 if unit_eps is None else unit_eps), _ptr(pos), _ptr(tok_slot), _ptr(k_pages), _ptr(v_pages),
         c_int64(page_stride), _ptr(page_table), page_table.shape[1], _ptr(q), DT[out_dtype], t, n_heads, n_kv_heads,
         head_dim, v_head_dim, q_dim, k_dim, v_dim, _stream()), "rope_norm_store")

@@ -80,8 +80,11 @@ class SigmoidAttention(Part):
             proj, col0 = ops.linear(h, self.w_in, out_dtype=torch.float32), 0
         inv_freq, rot, half = self._rotation()
         kv = view.as_tuple()
+        # the angles of the step's tokens: one table for all layers that rotate with these frequencies (the
+        # position part shares it through the step; a float32 model computes them where they are used)
+        table = self.position._table(ctx) if rot and hasattr(self.position, "_table") else None
         q = ops.rope_norm_store(proj, inv_freq, rot, half, self.unit_norm_eps, ctx.pos, ctx.tok_slot, kv, H, G, d, dv,
-                                self.k_dim, self.k_dim, self.v_dim, self.dtype, col0=col0)
+                                self.k_dim, self.k_dim, self.v_dim, self.dtype, col0=col0, cos_sin=table)
         if self.dtype == torch.float32:
             a = ops.sigmoid_attention(q, kv, ctx.pos, ctx.tok_slot, self.bias, H, G, self.k_dim, dv, self.v_dim,
                                       self.scale, self.window)
