@@ -769,18 +769,20 @@ __global__ __launch_bounds__(MAXT) void decay_carry_kernel(
     }
 }
 
-// ds: float32 [n_chunks, H, d, dv]; qa: the 16-bit type, [T, H, 32 * ceil(d / 32)]
+// ds: float32 [n_chunks, H, d, dv]; qa: the 16-bit type, [T, H, qa_dim] with qa_dim = 32 DBLK, DBLK the number of
+// 32-row blocks the kernels are compiled for (1, 2, 4 or 8: the next of these that holds d)
 extern "C" int li_decay_attn_chunked(const float* proj, int stride, int q_off, int k_off, int v_off, float* state,
                                      const float* decay, const int* seq_slot, const int* seq_qstart,
                                      const int* seq_qlen, const int* seq_chunk0, const int* chunk_seq,
-                                     const int* chunk_t0, int n_chunks, float* out, float* ds, void* qa, int n_seqs,
-                                     int H, int d, int dv, int dt, hipStream_t stream) {
+                                     const int* chunk_t0, int n_chunks, float* out, float* ds, void* qa, int qa_dim,
+                                     int n_seqs, int H, int d, int dv, int dt, hipStream_t stream) {
     if (n_seqs <= 0 || n_chunks <= 0) return LI_OK;
     if (H <= 0 || d <= 0 || dv <= 0 || dv > 256 || d > 256 || !seq_qstart || !seq_qlen || !seq_chunk0 || !chunk_seq ||
         !chunk_t0 || !ds || !qa)
         return LI_BAD_ARG;
     if (dt != DT_F16 && dt != DT_BF16) return LI_BAD_ARG;
     const int nw = (dv + 31) / 32, dblk = d <= 32 ? 1 : (d <= 64 ? 2 : (d <= 128 ? 4 : 8));
+    if (qa_dim != 32 * dblk) return LI_BAD_ARG;
     dim3 grid_a(n_chunks, H), block(64 * nw);
     const size_t lds = (size_t)(2 * 32 * (32 * dblk + 8) + 32 * (32 * nw + 8)) * 2 + 36 * sizeof(float);
 #define GO2(T, B, M)                                                                                             \

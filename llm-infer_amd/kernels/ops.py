@@ -1011,6 +1011,12 @@ def sigmoid_attention_decode(q, kv, seq_slot, seq_ctx, n_seqs, bias, n_heads, n_
 DECAY_CHUNK = 32        # tokens of one chunk of the chunked decay attention
 
 
+def decay_padded_dim(d: int) -> int:
+    """The width in which the chunked kernels hold a head of ``d`` dimensions: 32 times the number of 32-row
+    blocks they are compiled for (1, 2, 4 or 8), as csrc/mixers.hip li_decay_attn_chunked picks it."""
+    return 32 if d <= 32 else (64 if d <= 64 else (128 if d <= 128 else 256))
+
+
 def decay_chunk_lists(qlens) -> tuple:
     """The chunks of the chunked decay attention for sequences that bring ``qlens`` tokens: for every chunk its
     sequence and its first token within the sequence's tokens, and for every sequence its first chunk."""
@@ -1060,11 +1066,13 @@ def decay_attention(proj, q_off, k_off, v_off, state, decay, seq_slot, seq_qstar
               "the chunked kernels multiply 16-bit numbers and need the sequences' rows and the list of chunks")
         n_chunks = chunks["n_chunks"]
         ds = torch.empty((max(1, n_chunks), H, d, dv), dtype=torch.float32, device=proj.device)
-        qa = torch.empty((proj.shape[0], H, (d + 31) // 32 * 32), dtype=round_to, device=proj.device)
+        # q in 16 bits for the carry kernel, rows as wide as the kernels' template holds them: 32, 64, 128 or 256
+        # (the kernels index with that width; a narrower buffer would be written past its end)
+        qa = torch.empty((proj.shape[0], H, decay_padded_dim(d)), dtype=round_to, device=proj.device)
         _check(mixers().li_decay_attn_chunked(_ptr(proj), proj.shape[1], q_off, k_off, v_off, _ptr(state), _ptr(decay),
                                               _ptr(seq_slot), _ptr(seq_qstart), _ptr(seq_qlen), _ptr(chunks["seq_chunk0"]),
                                               _ptr(chunks["chunk_seq"]), _ptr(chunks["chunk_t0"]), n_chunks, _ptr(out),
-                                              _ptr(ds), _ptr(qa), n_seqs, H, d, dv, DT[round_to], _stream()),
+                                              _ptr(ds), _ptr(qa), qa.shape[2], n_seqs, H, d, dv, DT[round_to], _stream()),
                "decay_attn_chunked")
         return out
     _check(mixers().li_decay_attn(_ptr(proj), proj.shape[1], q_off, k_off, v_off, _ptr(state), _ptr(decay),

@@ -198,6 +198,8 @@ def test_chunk_lists_of_the_decay_attention():
     assert ops.DECAY_CHUNK == 32
     seq, t0, first = ops.decay_chunk_lists([70, 1, 32, 33])
     assert seq == [0, 0, 0, 1, 2, 3, 3] and t0 == [0, 32, 64, 0, 0, 0, 32] and first == [0, 3, 4, 5]
+    # the width of a head in the kernels: the next of 32, 64, 128, 256 (a head of 79 is held as 128, not as 96)
+    assert [ops.decay_padded_dim(d) for d in (1, 32, 33, 64, 65, 79, 96, 128, 129, 256)] == [32, 32, 64, 64, 128, 128, 128, 128, 256, 256]
 
 
 def test_default_slots_are_capped_by_the_states_memory():
