@@ -96,13 +96,21 @@ class KVGroup:
 
     def first_needed_page(self, length: int) -> int:
         """First page that a token at position ``length`` (the next one) still reads."""
-        if self.spec.window is None:
-            return 0
-        return max(0, length - self.spec.window + 1) // PAGE
+        first = 0
+        if self.spec.window is not None:
+            first = max(0, length - self.spec.window + 1)
+        if self.spec.block:
+            first = max(first, length - length % self.spec.block)
+        return first // PAGE
+
+    @property
+    def trims(self) -> bool:
+        """True if tokens leave what later tokens read (a window, blocks of positions)."""
+        return self.spec.window is not None or bool(self.spec.block)
 
     def reserve(self, slot: int, old_len: int, new_len: int, dirty: set, fresh: list, filled: bool = False) -> None:
         have = self.pages_of[slot]
-        lo = self.first_needed_page(old_len) if self.spec.window is not None else 0
+        lo = self.first_needed_page(old_len) if self.trims else 0
         want = range(lo, (new_len + PAGE - 1) // PAGE)
         need = [p for p in want if p not in have]
         if not need:
@@ -118,7 +126,7 @@ class KVGroup:
         dirty.add(slot)
 
     def release_outside_window(self, slot: int, length: int, dirty: set) -> None:
-        if self.spec.window is None:
+        if not self.trims:
             return
         first = self.first_needed_page(length)
         have = self.pages_of[slot]
@@ -284,7 +292,7 @@ class Cache:
 
     def trim_windows(self, slots) -> None:
         for g in self.groups:
-            if isinstance(g, KVGroup) and g.spec.window is not None:
+            if isinstance(g, KVGroup) and g.trims:
                 dirty = set()
                 for s in slots:
                     g.release_outside_window(s, self.lens[s], dirty)

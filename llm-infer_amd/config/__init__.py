@@ -1,5 +1,6 @@
 from .spec import PartSpec, SubLayerSpec, LayerSpec, ScheduleEntry, ModelSpec, ConfigError
 from .llama import LlamaConfig
 from .manirax import ManiraxConfig
+from .risonex import RisonexConfig
 
-__all__ = ["PartSpec", "SubLayerSpec", "LayerSpec", "ScheduleEntry", "ModelSpec", "ConfigError", "LlamaConfig", "ManiraxConfig"]
+__all__ = ["PartSpec", "SubLayerSpec", "LayerSpec", "ScheduleEntry", "ModelSpec", "ConfigError", "LlamaConfig", "ManiraxConfig", "RisonexConfig"]

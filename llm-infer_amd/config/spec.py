@@ -59,9 +59,12 @@ class LayerSpec:
 @dataclass(frozen=True)
 class ScheduleEntry:
     """One run of a layer.  ``cache_from`` names an earlier entry of the schedule whose
-    cache this run reads instead of keeping one of its own."""
+    cache this run reads instead of keeping one of its own.  ``before``: a part of the "stream" registry that
+    is run on the residual stream first (``forward(x, x0, ctx) -> x`` with x0 the embedding's output); entries
+    whose ``before`` specs are equal share one part, and so its tensors."""
     layer: int
     cache_from: int | None = None
+    before: PartSpec | None = None     # a "stream" part that rewrites the residual stream before this run
 
 
 @dataclass(frozen=True)

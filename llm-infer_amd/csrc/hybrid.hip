@@ -1,0 +1,564 @@
+// Kernels of hybrid decoders that alternate attention with a state-space mixer and route tokens to experts:
+// a scaled embedding with sinusoidal positions, the per-head RMS norm of q and k with the write into the paged
+// cache, differential attention over blocks of positions (two softmax maps over the same values, combined and
+// normed per head), the short causal convolution with its per-sequence history, the selective state-space
+// recurrence with a float32 state per sequence, the gated norm in groups behind it, plain activations, the
+// router of a mixture of experts and the weighting of the experts' hidden rows.  Every size is a run-time value.
+// Whatever a norm, a score, an attention weight, a decay, a step size or a recurrent state is made of is float32
+// here, whatever the type of the matrices.
+#include "common.h"
+
+__device__ __forceinline__ float sigmoidf_(float z) { return 1.f / (1.f + expf(-z)); }
+__device__ __forceinline__ float siluf_(float z) { return z / (1.f + expf(-z)); }
+__device__ __forceinline__ float softplusf_(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+__device__ __forceinline__ float gelu_erff_(float z) { return 0.5f * z * (1.f + erff(z * 0.70710678118654752f)); }
+
+#define DISPATCH_T(dt, CALL)                                     \
+    do {                                                         \
+        if ((dt) == DT_F32) { typedef float T; CALL; }           \
+        else if ((dt) == DT_F16) { typedef f16 T; CALL; }        \
+        else if ((dt) == DT_BF16) { typedef bf16 T; CALL; }      \
+        else return LI_BAD_ARG;                                  \
+    } while (0)
+
+// ---------------------------------------------------------------------------
+// x[t] = table[token[t]] * scale + P(pos[t]),  P(p)[2i] = sin(p f_i),  P(p)[2i+1] = cos(p f_i);  the
+// frequencies f_i come from the host (float32, one for every pair).  `freq` null: no positions are added.
+// ---------------------------------------------------------------------------
+template <class T>
+__global__ void embed_pos_kernel(const T* __restrict__ table, const int* __restrict__ tokens,
+                                 const int* __restrict__ pos, const float* __restrict__ freq, float* __restrict__ out,
+                                 int d, float scale) {
+    const int t = blockIdx.x;
+    const T* row = table + (int64_t)tokens[t] * d;
+    const float p = pos ? (float)pos[t] : 0.f;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+        float v = to_f32(row[i]) * scale;
+        if (freq) {
+            const float a = p * freq[i >> 1];
+            v += (i & 1) ? cosf(a) : sinf(a);
+        }
+        out[(int64_t)t * d + i] = v;
+    }
+}
+
+extern "C" int li_embed_pos(const void* table, int dt, const int* tokens, const int* pos, const float* freq, float* out,
+                            int n, int d, float scale, hipStream_t stream) {
+    if (n <= 0) return LI_OK;
+    if (d <= 0) return LI_BAD_ARG;
+    DISPATCH_T(dt, (embed_pos_kernel<T><<<n, 256, 0, stream>>>((const T*)table, tokens, pos, freq, out, d, scale)));
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// out[t] = [a[t] | b[t]] in type T (a, b float32 rows of width d): the input of a product over both.
+// ---------------------------------------------------------------------------
+template <class T>
+__global__ void concat_cast_kernel(const float* __restrict__ a, const float* __restrict__ b, T* __restrict__ out, int d) {
+    const int64_t t = blockIdx.x;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+        out[t * 2 * d + i] = from_f32<T>(a[t * d + i]);
+        out[t * 2 * d + d + i] = from_f32<T>(b[t * d + i]);
+    }
+}
+
+extern "C" int li_concat_cast(const float* a, const float* b, void* out, int dt, int n, int d, hipStream_t stream) {
+    if (n <= 0) return LI_OK;
+    DISPATCH_T(dt, (concat_cast_kernel<T><<<n, 256, 0, stream>>>(a, b, (T*)out, d)));
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// out = act(in), float32 in, type T out.  act: 0 gelu (erf), 1 gelu (tanh), 2 silu.
+// ---------------------------------------------------------------------------
+template <class T>
+__global__ void activation_kernel(const float* __restrict__ in, T* __restrict__ out, int64_t n, int act) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float z = in[i];
+    out[i] = from_f32<T>(act == 0 ? gelu_erff_(z) : (act == 1 ? gate_activation(z, true) : siluf_(z)));
+}
+
+extern "C" int li_activation(const float* in, void* out, int dt, int64_t n, int act, hipStream_t stream) {
+    if (n <= 0) return LI_OK;
+    if (act < 0 || act > 2) return LI_BAD_ARG;
+    DISPATCH_T(dt, (activation_kernel<T><<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(in, (T*)out, n, act)));
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// The cache of an attention whose keys are several maps wide.  A page holds PAGE tokens:
+//   keys   [kv head][token][KW]      KW = maps * d, the maps of a token side by side
+//   values [kv head][token][dv]      (the value part of a page is sized for dv rounded up to 32)
+// qk_norm_store: per token, from the float32 rows of the q/k/v product (columns q | k | v from `col0` on):
+// every map of every q and k head is divided by its root mean square over d and multiplied by a weight of size
+// d (null: none; eps < 0: no norm at all); q goes to `q_out` float32 [T, H, KW], k and v into the page of the
+// token's position.
+// ---------------------------------------------------------------------------
+struct MapPages {
+    void* k;
+    void* v;
+    int64_t page_stride;
+    const int* page_table;
+    int max_pages;
+};
+
+template <class T>
+__global__ void qk_norm_store_kernel(const float* __restrict__ qkv, int stride, int col0, const float* __restrict__ qw,
+                                     const float* __restrict__ kw, float eps, const int* __restrict__ pos,
+                                     const int* __restrict__ tok_slot, float* __restrict__ q_out, MapPages pg, int H,
+                                     int G, int maps, int d, int dv) {
+    const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const float* row = qkv + (int64_t)t * stride + col0;
+    const int KW = maps * d, p = pos[t];
+    const int page = pg.page_table[(int64_t)tok_slot[t] * pg.max_pages + p / PAGE], off = p % PAGE;
+    T* kp = (T*)pg.k + (int64_t)page * pg.page_stride;
+    T* vp = (T*)pg.v + (int64_t)page * pg.page_stride;
+    const int n_units = (H + G) * maps;                   // one wave a (head, map)
+    for (int u = wave; u < n_units; u += nw) {
+        const bool is_q = u < H * maps;
+        const float* src = row + (int64_t)u * d;          // q heads then k heads, each maps * d wide
+        float ss = 0.f;
+        for (int i = lane; i < d; i += 64) ss += src[i] * src[i];
+        const float r = eps >= 0.f ? 1.f / sqrtf(wave_sum(ss) / (float)d + eps) : 1.f;
+        const float* w = is_q ? qw : kw;
+        for (int i = lane; i < d; i += 64) {
+            const float v = src[i] * r * (w ? w[i] : 1.f);
+            if (is_q) q_out[(int64_t)t * H * KW + (int64_t)u * d + i] = v;
+            else {
+                const int ku = u - H * maps, g = ku / maps, m = ku - g * maps;
+                kp[((int64_t)g * PAGE + off) * KW + m * d + i] = from_f32<T>(v);
+            }
+        }
+    }
+    const float* vsrc = row + (int64_t)(H + G) * KW;
+    for (int i = threadIdx.x; i < G * dv; i += blockDim.x) {
+        const int g = i / dv, j = i - g * dv;
+        vp[((int64_t)g * PAGE + off) * dv + j] = from_f32<T>(vsrc[i]);
+    }
+}
+
+extern "C" int li_qk_norm_store(const float* qkv, int stride, int col0, const float* qw, const float* kw, float eps,
+                                const int* pos, const int* tok_slot, float* q_out, void* k_pages, void* v_pages,
+                                int64_t page_stride, const int* page_table, int max_pages, int dt, int n, int H, int G,
+                                int maps, int d, int dv, hipStream_t stream) {
+    if (n <= 0) return LI_OK;
+    if (H <= 0 || G <= 0 || maps <= 0 || d <= 0 || dv <= 0) return LI_BAD_ARG;
+    MapPages pg{k_pages, v_pages, page_stride, page_table, max_pages};
+    DISPATCH_T(dt, (qk_norm_store_kernel<T><<<n, 256, 0, stream>>>(qkv, stride, col0, qw, kw, eps, pos, tok_slot, q_out,
+                                                                  pg, H, G, maps, d, dv)));
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Differential attention over blocks of positions, one workgroup per (token, query head).
+// A token at position p sees the keys lo .. p with lo = p - p % block (block 0: lo = 0; window w > 0: lo is at
+// least p - w + 1).  Each of `maps` (1 or 2) maps is a softmax of its own over scores q_m . k_m * scale; with a_m
+// the maps' weighted sums of the SAME values,  o = a_1 - lambda a_2  (one map: o = a_1).  out_eps >= 0: o is
+// divided by its root mean square over dv and multiplied by out_scale.  Scores, weights, sums: float32.
+// The waves of the workgroup take the tiles of 64 keys in turn, a lane a key; each keeps a running maximum and
+// sum per map (online softmax) and its share of the output, and the shares are merged through LDS in wave order.
+// ---------------------------------------------------------------------------
+#define DA_WAVES 4
+#define DA_MAXV 4          // dv <= 64 * DA_MAXV
+
+template <class T, int MAPS>
+__global__ __launch_bounds__(64 * DA_WAVES) void diff_attn_kernel(
+    const float* __restrict__ q, T* __restrict__ out, MapPages pg, const int* __restrict__ pos,
+    const int* __restrict__ tok_slot, int H, int G, int d, int dv, float scale, int block, int window, float lambda,
+    float out_eps, float out_scale) {
+    extern __shared__ float lds[];
+    const int KW = MAPS * d;
+    float* sq = lds;                                   // [KW]
+    float* sm = sq + KW;                               // [DA_WAVES][MAPS] maxima
+    float* sl = sm + DA_WAVES * MAPS;                  // [DA_WAVES][MAPS] sums
+    float* so = sl + DA_WAVES * MAPS;                  // [DA_WAVES][MAPS][dv]
+    __shared__ float scratch[16];
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int g = h / (H / G), p = pos[t];
+    int lo = block > 0 ? p - p % block : 0;
+    if (window > 0) lo = max(lo, p - window + 1);
+    for (int i = threadIdx.x; i < KW; i += blockDim.x) sq[i] = q[((int64_t)t * H + h) * KW + i];
+    __syncthreads();
+    const int* table = pg.page_table + (int64_t)tok_slot[t] * pg.max_pages;
+    float m[MAPS], l[MAPS], o[MAPS][DA_MAXV];
+#pragma unroll
+    for (int a = 0; a < MAPS; ++a) {
+        m[a] = -INFINITY; l[a] = 0.f;
+#pragma unroll
+        for (int c = 0; c < DA_MAXV; ++c) o[a][c] = 0.f;
+    }
+    const int n_tiles = (p - lo) / 64 + 1;
+    for (int tile = wave; tile < n_tiles; tile += DA_WAVES) {
+        const int j = lo + tile * 64 + lane;           // this lane's key
+        float s[MAPS];
+        const T* krow = nullptr;
+        if (j <= p) krow = (const T*)pg.k + (int64_t)table[j / PAGE] * pg.page_stride + ((int64_t)g * PAGE + j % PAGE) * KW;
+#pragma unroll
+        for (int a = 0; a < MAPS; ++a) {
+            float acc = 0.f;
+            if (krow) for (int i = 0; i < d; ++i) acc += sq[a * d + i] * to_f32(krow[a * d + i]);
+            s[a] = krow ? acc * scale : -INFINITY;
+        }
+        float pw[MAPS];
+#pragma unroll
+        for (int a = 0; a < MAPS; ++a) {
+            const float mt = fmaxf(m[a], wave_max(s[a]));          // lane 0's key is always visible: finite
+            const float f = expf(m[a] - mt);                       // 0 the first time (m = -inf)
+            pw[a] = krow ? expf(s[a] - mt) : 0.f;
+            l[a] = l[a] * f + wave_sum(pw[a]);
+            m[a] = mt;
+#pragma unroll
+            for (int c = 0; c < DA_MAXV; ++c) o[a][c] *= f;
+        }
+        const int n_keys = min(64, p - (lo + tile * 64) + 1);
+        for (int kk = 0; kk < n_keys; ++kk) {
+            const int jj = lo + tile * 64 + kk;
+            const T* vrow = (const T*)pg.v + (int64_t)table[jj / PAGE] * pg.page_stride + ((int64_t)g * PAGE + jj % PAGE) * dv;
+            float w[MAPS];
+#pragma unroll
+            for (int a = 0; a < MAPS; ++a) w[a] = __shfl(pw[a], kk, WAVE);
+#pragma unroll
+            for (int c = 0; c < DA_MAXV; ++c) {
+                const int i = lane + 64 * c;
+                if (i < dv) {
+                    const float v = to_f32(vrow[i]);
+#pragma unroll
+                    for (int a = 0; a < MAPS; ++a) o[a][c] += w[a] * v;
+                }
+            }
+        }
+    }
+    // merge the waves' shares in wave order
+#pragma unroll
+    for (int a = 0; a < MAPS; ++a) {
+        if (lane == 0) { sm[wave * MAPS + a] = m[a]; sl[wave * MAPS + a] = l[a]; }
+#pragma unroll
+        for (int c = 0; c < DA_MAXV; ++c) {
+            const int i = lane + 64 * c;
+            if (i < dv) so[(wave * MAPS + a) * dv + i] = o[a][c];
+        }
+    }
+    __syncthreads();
+    float ss = 0.f;
+    float res[DA_MAXV];
+#pragma unroll
+    for (int c = 0; c < DA_MAXV; ++c) res[c] = 0.f;
+    if (wave == 0) {
+#pragma unroll
+        for (int c = 0; c < DA_MAXV; ++c) {
+            const int i = lane + 64 * c;
+            if (i < dv) {
+                float am[MAPS];
+#pragma unroll
+                for (int a = 0; a < MAPS; ++a) {
+                    float M = sm[a];
+                    for (int w = 1; w < DA_WAVES; ++w) M = fmaxf(M, sm[w * MAPS + a]);
+                    float L = 0.f, O = 0.f;
+                    for (int w = 0; w < DA_WAVES; ++w) {
+                        const float mw = sm[w * MAPS + a];
+                        const float f = mw == -INFINITY ? 0.f : expf(mw - M);
+                        L += sl[w * MAPS + a] * f;
+                        O += so[(w * MAPS + a) * dv + i] * f;
+                    }
+                    am[a] = O / L;
+                }
+                res[c] = MAPS == 2 ? am[0] - lambda * am[MAPS - 1] : am[0];
+                ss += res[c] * res[c];
+            }
+        }
+    }
+    float r = out_scale;
+    if (out_eps >= 0.f) r = out_scale / sqrtf(block_sum(ss, scratch) / (float)dv + out_eps);   // waves 1.. add 0
+    if (wave == 0) {
+#pragma unroll
+        for (int c = 0; c < DA_MAXV; ++c) {
+            const int i = lane + 64 * c;
+            if (i < dv) out[((int64_t)t * H + h) * dv + i] = from_f32<T>(res[c] * r);
+        }
+    }
+}
+
+extern "C" int li_diff_attn(const float* q, void* out, int dt, void* k_pages, void* v_pages, int64_t page_stride,
+                            const int* page_table, int max_pages, const int* pos, const int* tok_slot, int n, int H, int G,
+                            int maps, int d, int dv, float scale, int block, int window, float lambda, float out_eps,
+                            float out_scale, hipStream_t stream) {
+    if (n <= 0) return LI_OK;
+    if (H <= 0 || G <= 0 || H % G || d <= 0 || dv <= 0 || block < 0 || window < 0) return LI_BAD_ARG;
+    if (maps < 1 || maps > 2 || dv > 64 * DA_MAXV) return LI_UNSUPPORTED;
+    MapPages pg{k_pages, v_pages, page_stride, page_table, max_pages};
+    dim3 grid(n, H), blk(64 * DA_WAVES);
+    const size_t lds = (size_t)(maps * d + 2 * DA_WAVES * maps + DA_WAVES * maps * dv) * sizeof(float);
+    if (lds > 60000) return LI_UNSUPPORTED;
+#define GO(M) diff_attn_kernel<T, M><<<grid, blk, lds, stream>>>(q, (T*)out, pg, pos, tok_slot, H, G, d, dv, scale, block, \
+                                                                 window, lambda, out_eps, out_scale)
+    DISPATCH_T(dt, { if (maps == 1) GO(1); else GO(2); });
+#undef GO
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// A short causal convolution per channel with its activation:
+//   out[t][c] = silu(b[c] + sum over j < taps of w[c][j] u[t - (taps - 1 - j)][c])
+// u are `channels` columns of the float32 rows `in` from column `col0` on.  Inputs before the first token that a
+// sequence brings to this step come from its history `hist` [slots, taps - 1, channels] (the last taps - 1 inputs
+// of the steps before, oldest first); before position 0 they are zero.  conv_history_kernel then leaves every
+// sequence's last taps - 1 inputs there.
+// ---------------------------------------------------------------------------
+#define CONV_MAX_TAPS 16
+
+__global__ void conv_silu_kernel(const float* __restrict__ in, int stride, int col0, const float* __restrict__ w,
+                                 const float* __restrict__ b, const float* __restrict__ hist, const int* __restrict__ pos,
+                                 const int* __restrict__ tok_slot, float* __restrict__ out, int channels, int taps) {
+    const int t = blockIdx.x, p = pos[t], slot = tok_slot[t];
+    // how many tokens before this one its sequence has in this step (at most taps - 1 matter)
+    int inside = 0;
+    while (inside < taps - 1 && t - inside - 1 >= 0 && tok_slot[t - inside - 1] == slot) ++inside;
+    const float* h = hist + (int64_t)slot * (taps - 1) * channels;
+    for (int c = threadIdx.x; c < channels; c += blockDim.x) {
+        float acc = b ? b[c] : 0.f;
+        for (int back = 0; back < taps; ++back) {                  // back = taps - 1 - j
+            float u = 0.f;
+            if (back <= inside) u = in[(int64_t)(t - back) * stride + col0 + c];
+            else if (p - back >= 0) u = h[(int64_t)(taps - 1 - (back - inside)) * channels + c];
+            acc += w[(int64_t)c * taps + (taps - 1 - back)] * u;
+        }
+        out[(int64_t)t * channels + c] = siluf_(acc);
+    }
+}
+
+__global__ void conv_history_kernel(const float* __restrict__ in, int stride, int col0, float* __restrict__ hist,
+                                    const int* __restrict__ seq_slot, const int* __restrict__ seq_qstart,
+                                    const int* __restrict__ seq_qlen, int channels, int taps) {
+    const int seq = blockIdx.x;
+    const int q0 = seq_qstart ? seq_qstart[seq] : seq, n = seq_qlen ? seq_qlen[seq] : 1;
+    float* h = hist + (int64_t)seq_slot[seq] * (taps - 1) * channels;
+    for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < channels; c += gridDim.y * blockDim.x) {
+        float keep[CONV_MAX_TAPS];
+        for (int r = 0; r < taps - 1; ++r) {
+            const int back = taps - 1 - r;                          // row r holds the input `back` tokens before the next
+            keep[r] = back <= n ? in[(int64_t)(q0 + n - back) * stride + col0 + c] : h[(int64_t)(r + n) * channels + c];
+        }
+        for (int r = 0; r < taps - 1; ++r) h[(int64_t)r * channels + c] = keep[r];
+    }
+}
+
+extern "C" int li_conv_silu(const float* in, int stride, int col0, const float* w, const float* b, float* hist,
+                            const int* pos, const int* tok_slot, const int* seq_slot, const int* seq_qstart,
+                            const int* seq_qlen, float* out, int n_tokens, int n_seqs, int channels, int taps,
+                            hipStream_t stream) {
+    if (n_tokens <= 0) return LI_OK;
+    if (channels <= 0 || taps < 1 || taps > CONV_MAX_TAPS) return LI_BAD_ARG;
+    conv_silu_kernel<<<n_tokens, 256, 0, stream>>>(in, stride, col0, w, b, hist, pos, tok_slot, out, channels, taps);
+    if (taps > 1) {
+        dim3 grid(n_seqs, (channels + 255) / 256);
+        conv_history_kernel<<<grid, 256, 0, stream>>>(in, stride, col0, hist, seq_slot, seq_qstart, seq_qlen, channels, taps);
+    }
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// The selective state-space recurrence.  Per sequence and head h (group g = h / (P / G)), with x_t [dv],
+// B_t, C_t [N] from the rows `xbc` (columns x | B | C) and the raw step size from `proj` column dt_col + h:
+//   dt = softplus(raw + dt_bias[h]);   a = exp(-exp(A_log[h]) dt)
+//   S <- a S + dt B_t x_t^T   (S is N x dv, float32, kept for every sequence in `state` [slots, P, N, dv])
+//   y_t = S^T C_t + D[h] x_t
+// One wave per (sequence, head, 64 columns of dv): a lane keeps its column of S in registers for all the tokens
+// that the sequence brings; B_t and C_t reach the lanes through LDS, fetched a token ahead.
+// ---------------------------------------------------------------------------
+template <int NMAX>
+__global__ __launch_bounds__(64) void ssm_scan_kernel(
+    const float* __restrict__ xbc, int xbc_stride, const float* __restrict__ proj, int proj_stride, int dt_col,
+    const float* __restrict__ dt_bias, const float* __restrict__ A_log, const float* __restrict__ D,
+    float* __restrict__ state, const int* __restrict__ seq_slot, const int* __restrict__ seq_qstart,
+    const int* __restrict__ seq_qlen, float* __restrict__ y, int P, int G, int N, int dv) {
+    __shared__ float sb[2][2 * NMAX];                       // [stage][B | C]
+    const int seq = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, col = blockIdx.z * 64 + lane;
+    const int g = h / (P / G), inner = P * dv;
+    const int q0 = seq_qstart ? seq_qstart[seq] : seq, n = seq_qlen ? seq_qlen[seq] : 1;
+    const bool live = col < dv;
+    float* S = state + (((int64_t)seq_slot[seq] * P + h) * N) * dv + col;
+    float s[NMAX];
+#pragma unroll
+    for (int i = 0; i < NMAX; ++i) s[i] = (live && i < N) ? S[(int64_t)i * dv] : 0.f;
+    const float negA = -expf(A_log[h]), bias = dt_bias[h], dh = D ? D[h] : 0.f;
+    const int b_off = inner + g * N, c_off = inner + G * N + g * N;
+    auto fetch = [&](int t, int stage) {
+        const float* row = xbc + (int64_t)(q0 + t) * xbc_stride;
+        for (int i = lane; i < N; i += 64) { sb[stage][i] = row[b_off + i]; sb[stage][NMAX + i] = row[c_off + i]; }
+    };
+    if (n > 0) fetch(0, 0);
+    __syncthreads();
+    for (int t = 0; t < n; ++t) {
+        const int stage = t & 1;
+        if (t + 1 < n) fetch(t + 1, stage ^ 1);
+        const float dt = softplusf_(proj[(int64_t)(q0 + t) * proj_stride + dt_col + h] + bias);
+        const float a = expf(negA * dt);
+        const float x = live ? xbc[(int64_t)(q0 + t) * xbc_stride + h * dv + col] : 0.f;
+        const float dx = dt * x;
+        float acc = 0.f;
+#pragma unroll
+        for (int i = 0; i < NMAX; ++i) {
+            if (i < N) {
+                s[i] = a * s[i] + sb[stage][i] * dx;
+                acc += s[i] * sb[stage][NMAX + i];
+            }
+        }
+        if (live) y[(int64_t)(q0 + t) * inner + h * dv + col] = acc + dh * x;
+        __syncthreads();
+    }
+    if (live) {
+#pragma unroll
+        for (int i = 0; i < NMAX; ++i) if (i < N) S[(int64_t)i * dv] = s[i];
+    }
+}
+
+extern "C" int li_ssm_scan(const float* xbc, int xbc_stride, const float* proj, int proj_stride, int dt_col,
+                           const float* dt_bias, const float* A_log, const float* D, float* state, const int* seq_slot,
+                           const int* seq_qstart, const int* seq_qlen, float* y, int n_seqs, int P, int G, int N, int dv,
+                           hipStream_t stream) {
+    if (n_seqs <= 0) return LI_OK;
+    if (P <= 0 || G <= 0 || P % G || N <= 0 || dv <= 0) return LI_BAD_ARG;
+    if (N > 256) return LI_UNSUPPORTED;
+    dim3 grid(n_seqs, P, (dv + 63) / 64);
+#define GO(NM) ssm_scan_kernel<NM><<<grid, 64, 0, stream>>>(xbc, xbc_stride, proj, proj_stride, dt_col, dt_bias, A_log, D, \
+                                                            state, seq_slot, seq_qstart, seq_qlen, y, P, G, N, dv)
+    if (N <= 16) GO(16); else if (N <= 32) GO(32); else if (N <= 64) GO(64); else if (N <= 128) GO(128); else GO(256);
+#undef GO
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// out = N_g(y * silu(z)) * w: the gate first, then each of `groups` equal parts of a row divided by its own
+// root mean square.  y float32 [T, n]; z: n columns of the float32 rows `zrows` from column z_col on.
+// ---------------------------------------------------------------------------
+template <class T>
+__global__ void gated_group_norm_kernel(const float* __restrict__ y, const float* __restrict__ zrows, int z_stride,
+                                        int z_col, const float* __restrict__ w, T* __restrict__ out, int n, int groups,
+                                        float eps) {
+    __shared__ float scratch[16];
+    const int t = blockIdx.x, grp = blockIdx.y, part = n / groups;
+    const float* yr = y + (int64_t)t * n + grp * part;
+    const float* zr = zrows + (int64_t)t * z_stride + z_col + grp * part;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < part; i += blockDim.x) { const float v = yr[i] * siluf_(zr[i]); ss += v * v; }
+    const float r = 1.f / sqrtf(block_sum(ss, scratch) / (float)part + eps);
+    for (int i = threadIdx.x; i < part; i += blockDim.x)
+        out[(int64_t)t * n + grp * part + i] = from_f32<T>(yr[i] * siluf_(zr[i]) * r * w[grp * part + i]);
+}
+
+extern "C" int li_gated_group_norm(const float* y, const float* zrows, int z_stride, int z_col, const float* w, void* out,
+                                   int dt, int n_rows, int n, int groups, float eps, hipStream_t stream) {
+    if (n_rows <= 0) return LI_OK;
+    if (n <= 0 || groups <= 0 || n % groups) return LI_BAD_ARG;
+    dim3 grid(n_rows, groups);
+    DISPATCH_T(dt, (gated_group_norm_kernel<T><<<grid, 256, 0, stream>>>(y, zrows, z_stride, z_col, w, (T*)out, n, groups, eps)));
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// The router of a mixture of experts, one wave per token.  `logits` float32 [T, n_cols]: n_route router outputs,
+// then (has_gate 1) one column whose sigmoid weighs an expert that every token uses (has_gate 2: its weight is 1).  s = softmax over the n_route
+// outputs; the `top` outputs with the largest s + correction are chosen (the first of equals); their weights are
+// s / (sum of the chosen s + 1e-20) * route_scale.  The first n_real outputs are experts with matrices: their
+// weights (0 where not chosen) go to `weights` [T, n_real (+ 1)], the gate's sigmoid into the last column.  The
+// outputs behind them pass the token's input on: residual[t] += (sum of their weights) * h[t].
+// ---------------------------------------------------------------------------
+template <class T>
+__global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__ logits, int n_cols,
+                                                       const float* __restrict__ correction, const T* __restrict__ h,
+                                                       float* __restrict__ residual, float* __restrict__ weights,
+                                                       int width, int n_route, int n_real, int top, int has_gate,
+                                                       float route_scale) {
+    extern __shared__ float lds[];
+    float* s = lds;                      // [n_route] softmax scores
+    float* c = s + n_route;              // [n_route] choice scores, -inf once chosen
+    const int t = blockIdx.x, lane = threadIdx.x;
+    const float* z = logits + (int64_t)t * n_cols;
+    float mx = -INFINITY;
+    for (int i = lane; i < n_route; i += 64) mx = fmaxf(mx, z[i]);
+    mx = wave_max(mx);
+    float sum = 0.f;
+    for (int i = lane; i < n_route; i += 64) { const float e = expf(z[i] - mx); s[i] = e; sum += e; }
+    sum = wave_sum(sum);
+    const int wcols = n_real + (has_gate ? 1 : 0);
+    for (int i = lane; i < n_route; i += 64) {
+        s[i] /= sum;
+        c[i] = s[i] + (correction ? correction[i] : 0.f);
+    }
+    for (int i = lane; i < wcols; i += 64) weights[(int64_t)t * wcols + i] = 0.f;
+    __syncthreads();
+    float chosen_sum = 0.f;
+    for (int k = 0; k < top; ++k) {
+        float best = -INFINITY; int bi = 0x7fffffff;
+        for (int i = lane; i < n_route; i += 64) if (c[i] > best) { best = c[i]; bi = i; }
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ob = __shfl_xor(best, o, WAVE); const int oi = __shfl_xor(bi, o, WAVE);
+            if (ob > best || (ob == best && oi < bi)) { best = ob; bi = oi; }
+        }
+        chosen_sum += s[bi];
+        __syncthreads();
+        if (lane == 0) c[bi] = -INFINITY;
+        __syncthreads();
+    }
+    const float f = route_scale / (chosen_sum + 1e-20f);
+    float pass = 0.f;                    // the weight of the outputs that pass the input on
+    // every lane knows the chosen set through c == -inf
+    for (int i = lane; i < n_route; i += 64) {
+        if (c[i] == -INFINITY) {
+            const float w = s[i] * f;
+            if (i < n_real) weights[(int64_t)t * wcols + i] = w; else pass += w;
+        }
+    }
+    pass = wave_sum(pass);
+    if (has_gate && lane == 0) weights[(int64_t)t * wcols + n_real] = has_gate == 2 ? 1.f : sigmoidf_(z[n_route]);
+    if (pass != 0.f)
+        for (int i = lane; i < width; i += 64) residual[(int64_t)t * width + i] += pass * to_f32(h[(int64_t)t * width + i]);
+}
+
+extern "C" int li_moe_route(const float* logits, int n_cols, const float* correction, const void* h, int dt,
+                            float* residual, float* weights, int n, int width, int n_route, int n_real, int top,
+                            int has_gate, float route_scale, hipStream_t stream) {
+    if (n <= 0) return LI_OK;
+    if (n_route <= 0 || n_real < 0 || n_real > n_route || top < 1 || top > n_route || n_cols < n_route + (has_gate == 1 ? 1 : 0) ||
+        has_gate < 0 || has_gate > 2)
+        return LI_BAD_ARG;
+    if (n_route > 4096) return LI_UNSUPPORTED;
+    const size_t lds = (size_t)2 * n_route * sizeof(float);
+    DISPATCH_T(dt, (moe_route_kernel<T><<<n, 64, lds, stream>>>(logits, n_cols, correction, (const T*)h, residual, weights,
+                                                                 width, n_route, n_real, top, has_gate, route_scale)));
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// The experts' hidden rows side by side, t [T, n_blocks * ff + tail]: block e of a row is multiplied by
+// weights[t][e], the tail (an expert of another width that every token uses) by weights[t][n_blocks].
+// ---------------------------------------------------------------------------
+template <class T>
+__global__ void scale_blocks_kernel(T* __restrict__ t, const float* __restrict__ weights, int n_blocks, int ff, int tail) {
+    const int64_t row = blockIdx.x;
+    const int cols = n_blocks * ff + tail, wcols = n_blocks + (tail ? 1 : 0);
+    for (int i = threadIdx.x; i < cols; i += blockDim.x) {
+        const int e = i < n_blocks * ff ? i / ff : n_blocks;
+        const float w = weights[row * wcols + e];
+        t[row * cols + i] = from_f32<T>(w == 0.f ? 0.f : to_f32(t[row * cols + i]) * w);
+    }
+}
+
+extern "C" int li_scale_blocks(void* t, int dt, const float* weights, int n, int n_blocks, int ff, int tail,
+                               hipStream_t stream) {
+    if (n <= 0) return LI_OK;
+    if (n_blocks < 0 || ff < 0 || tail < 0) return LI_BAD_ARG;
+    DISPATCH_T(dt, (scale_blocks_kernel<T><<<n, 256, 0, stream>>>((T*)t, weights, n_blocks, ff, tail)));
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}

@@ -7,6 +7,7 @@ import torch
 
 from .. import parts as _parts  # noqa: F401  (registers the built-in parts)
 from ..config.spec import ModelSpec
+from ..kernels import ops
 from ..parts.base import Part, cache_specs_of, collect_params
 from ..parts.block import SubLayer
 from ..registry import lookup
@@ -40,6 +41,14 @@ class DecoderModel(Part):
                                      None if sub.post_norm is None else _make("norm", sub.post_norm, dtype, dev)))
             self.layers.append(lookup("block", ls.block)(subs, **ls.block_params))
             self.layer_mixers.append(mixers)
+        # parts that rewrite the residual stream before a run of a layer; equal specs share one part
+        self.stream_parts, self._before = {}, []
+        for e in spec.schedule:
+            b = getattr(e, "before", None)
+            key = None if b is None else (b.kind, b.prefix, repr(sorted(b.params.items())))
+            if key is not None and key not in self.stream_parts:
+                self.stream_parts[key] = _make("stream", b, dtype, dev)
+            self._before.append(key)
         self.final_norm = _make("norm", spec.final_norm, dtype, dev)
         self.head = _make("head", spec.head, dtype, dev)
         self.schedule = list(spec.schedule)
@@ -68,7 +77,8 @@ class DecoderModel(Part):
 
     # -- weights -----------------------------------------------------------
     def children(self):
-        return [self.embedding, *self.positions.values(), *self.layers, self.final_norm, self.head]
+        return [self.embedding, *self.positions.values(), *self.stream_parts.values(), *self.layers, self.final_norm,
+                self.head]
 
     def recordable(self) -> bool:
         """True if every part's forward pass can be recorded into a graph."""
@@ -123,8 +133,12 @@ class DecoderModel(Part):
     # -- the forward pass of one step ---------------------------------------
     def forward(self, ctx, cache) -> torch.Tensor:
         """Runs the step's tokens through the schedule; returns float32 logits [n_want, vocab]."""
-        x = self.embedding.forward(ctx)
+        x = x0 = self.embedding.forward(ctx)
         for i, e in enumerate(self.schedule):
+            if self._before[i] is not None:
+                x = self.stream_parts[self._before[i]].forward(x, x0, ctx)       # a new tensor: x0 stays as it is
+            elif x is x0 and self.stream_parts:
+                x = ops.copy_rows(x0)            # the layers add in place, and a later part reads the embedding's output
             owner = i if e.cache_from is None else e.cache_from
             # one view for a mixer, or the list of its views for one that asks several things of the cache
             views = [[cache.view(u) for u in self._unit[owner, k]] if multi else cache.view(self._unit[owner, k][0])

@@ -191,6 +191,15 @@ def mixers_library(force=False):
     return _load("libli_mixers.so", MIXER_SOURCES, (), force)
 
 
+HYBRID_SOURCES = ("hybrid.hip",)
+
+
+def hybrid_library(force=False):
+    """The kernels of hybrid decoders (csrc/hybrid.hip: differential attention over blocks of positions, the
+    state-space recurrence and its convolution, the experts' router): a library of its own, as the mixers' is."""
+    return _load("libli_hybrid.so", HYBRID_SOURCES, (), force)
+
+
 SIGMOID_ATTN_SOURCE = "sigmoid_attention.hip"
 
 
@@ -213,6 +222,7 @@ def build_all(head_dims=(16, 32, 48, 64, 128), force=True, sigmoid_head_dims=((4
     sigmoid attention library for each pair of head sizes given."""
     core_library(force=force)
     mixers_library(force=force)
+    hybrid_library(force=force)
     with ThreadPoolExecutor(max_workers=4) as pool:
         list(pool.map(lambda p: _build_library(*_sigmoid_attention_args(*p), force), sigmoid_head_dims))
     with ThreadPoolExecutor(max_workers=4) as pool:

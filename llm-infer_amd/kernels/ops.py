@@ -1106,3 +1106,209 @@ def polynorm(z, coef, eps, out_dtype) -> torch.Tensor:
     _check(mixers().li_polynorm(_ptr(z), _ptr(coef), _ptr(out), DT[out_dtype], z.shape[0], z.shape[1], c_float(eps),
                                 _stream()), "polynorm")
     return out
+
+
+# ---------------------------------------------------------------------------
+# hybrid decoders (csrc/hybrid.hip): differential attention over blocks of positions, the state-space mixer,
+# routed experts, a scaled embedding with sinusoidal positions
+# ---------------------------------------------------------------------------
+_hybrid = None
+ACTIVATIONS = {"gelu": 0, "gelu_tanh": 1, "silu": 2}
+
+
+def hybrid():
+    global _hybrid
+    if _hybrid is None:
+        _hybrid = build.hybrid_library()
+    return _hybrid
+
+
+def _i32(t, n, what):
+    _need(t is not None and t.dtype == torch.int32 and t.numel() >= n, f"{what}: int32, one for each of {n}")
+
+
+def embed_positions(table, tokens, pos, freq, scale: float) -> torch.Tensor:
+    """x[t] = float32(table[tokens[t]]) * scale + P(pos[t]); P(p)[2i] = sin(p freq[i]), P(p)[2i+1] = cos(p freq[i])
+    (``freq`` None: no positions)."""
+    _dev(table, tokens, pos, freq)
+    n, (vocab, d) = tokens.numel(), table.shape
+    _need(tokens.dtype == torch.int32 and table.dim() == 2 and table.dtype in DT, "embed: int32 tokens, a float table")
+    if freq is not None:
+        _i32(pos, n, "embed positions")
+        _need(freq.dtype == torch.float32 and freq.numel() >= (d + 1) // 2, "embed: a float32 frequency for every pair")
+    out = torch.empty((n, d), dtype=torch.float32, device=table.device)
+    _check(hybrid().li_embed_pos(_ptr(table), DT[table.dtype], _ptr(tokens), _ptr(pos), _ptr(freq), _ptr(out), n, d,
+                                 c_float(scale), _stream()), "embed_pos")
+    return out
+
+
+def concat_cast(a, b, dtype) -> torch.Tensor:
+    """[a | b] row by row in ``dtype`` (a, b float32 of one shape)."""
+    _dev(a, b)
+    _f32_rows(a, "concat a")
+    _need(b.dtype == torch.float32 and b.shape == a.shape and dtype in DT, "concat: two float32 tensors of one shape")
+    out = torch.empty((a.shape[0], 2 * a.shape[1]), dtype=dtype, device=a.device)
+    _check(hybrid().li_concat_cast(_ptr(a), _ptr(b), _ptr(out), DT[dtype], a.shape[0], a.shape[1], _stream()), "concat_cast")
+    return out
+
+
+def activation(z, kind: str, out_dtype) -> torch.Tensor:
+    """act(z) for float32 z in ``out_dtype``; kind: gelu (erf), gelu_tanh, silu."""
+    _dev(z)
+    _need(z.dtype == torch.float32 and kind in ACTIVATIONS and out_dtype in DT, f"activation {kind!r}: float32 in, gelu/gelu_tanh/silu")
+    out = torch.empty(z.shape, dtype=out_dtype, device=z.device)
+    _check(hybrid().li_activation(_ptr(z), _ptr(out), DT[out_dtype], c_int64(z.numel()), ACTIVATIONS[kind], _stream()),
+           "activation")
+    return out
+
+
+def _map_pages_check(kv, n_kv_heads, key_width, v_dim):
+    k_pages, v_pages, page_stride, page_table = kv
+    _dev(k_pages, v_pages, page_table)
+    _need(k_pages.dtype == v_pages.dtype and k_pages.dtype in DT, "cache: one float type for keys and values")
+    _need(page_table.dtype == torch.int32 and page_table.dim() == 2, "page_table: int32 [slots, pages]")
+    _need(page_stride >= n_kv_heads * PAGE * (key_width + v_dim), "a page is too small for these keys and values")
+    return k_pages, v_pages, page_stride, page_table
+
+
+def qk_norm_store(qkv, col0, q_weight, k_weight, eps, pos, tok_slot, kv, n_heads, n_kv_heads, maps, d, dv) -> torch.Tensor:
+    """From the float32 rows of a q/k/v product (columns from ``col0``: q [H, maps, d] | k [G, maps, d] | v [G, dv]):
+    each map of each q and k head divided by its root mean square over d and multiplied by a weight [d] (``eps``
+    None: no norm); returns q float32 [T, H, maps * d]; k and v go into the pages (keys [head][token][maps * d],
+    values [head][token][dv]) at each token's position."""
+    _dev(qkv, q_weight, k_weight, pos, tok_slot)
+    _f32_rows(qkv, "qk_norm_store rows")
+    t = qkv.shape[0]
+    kw = maps * d
+    _need(col0 >= 0 and col0 + (n_heads + n_kv_heads) * kw + n_kv_heads * dv <= qkv.shape[1], "qk_norm_store: columns beyond the rows")
+    for w in (q_weight, k_weight):
+        _need(w is None or (w.dtype == torch.float32 and w.shape == (d,)), "q/k norm weight: float32 [d]")
+    _i32(pos, t, "positions")
+    _i32(tok_slot, t, "slots")
+    k_pages, v_pages, page_stride, page_table = _map_pages_check(kv, n_kv_heads, kw, dv)
+    q = torch.empty((t, n_heads, kw), dtype=torch.float32, device=qkv.device)
+    _check(hybrid().li_qk_norm_store(_ptr(qkv), qkv.shape[1], col0, _ptr(q_weight), _ptr(k_weight),
+                                     c_float(-1.0 if eps is None else eps), _ptr(pos), _ptr(tok_slot), _ptr(q), _ptr(k_pages),
+                                     _ptr(v_pages), c_int64(page_stride), _ptr(page_table), page_table.shape[1],
+                                     DT[k_pages.dtype], t, n_heads, n_kv_heads, maps, d, dv, _stream()), "qk_norm_store")
+    return q
+
+
+def diff_attention(q, kv, pos, tok_slot, n_heads, n_kv_heads, maps, d, dv, scale, block, window, lam, out_eps, out_scale,
+                   out_dtype) -> torch.Tensor:
+    """Attention of ``maps`` softmax maps (1 or 2) over the same values: o = a_1 - lam a_2, then (``out_eps`` not
+    None) o divided by its root mean square over dv, times ``out_scale``.  A token at position p sees the keys
+    from p - p % block on (``block`` 0: from 0; ``window`` w: at most the last w).  q float32 [T, H, maps * d];
+    returns [T, H * dv] in ``out_dtype``."""
+    _dev(q, pos, tok_slot)
+    t = q.shape[0]
+    _need(q.dtype == torch.float32 and q.shape == (t, n_heads, maps * d), "q: float32 [T, H, maps * d]")
+    _need(maps in (1, 2) and dv <= 256 and n_heads % n_kv_heads == 0, "diff_attention: one or two maps, values up to 256 wide")
+    _i32(pos, t, "positions")
+    _i32(tok_slot, t, "slots")
+    k_pages, v_pages, page_stride, page_table = _map_pages_check(kv, n_kv_heads, maps * d, dv)
+    _need(out_dtype == k_pages.dtype, "diff_attention: the output has the cache's type")
+    out = torch.empty((t, n_heads * dv), dtype=out_dtype, device=q.device)
+    _check(hybrid().li_diff_attn(_ptr(q), _ptr(out), DT[out_dtype], _ptr(k_pages), _ptr(v_pages), c_int64(page_stride),
+                                 _ptr(page_table), page_table.shape[1], _ptr(pos), _ptr(tok_slot), t, n_heads, n_kv_heads,
+                                 maps, d, dv, c_float(scale), int(block or 0), int(window or 0), c_float(lam),
+                                 c_float(-1.0 if out_eps is None else out_eps), c_float(out_scale), _stream()), "diff_attn")
+    return out
+
+
+def conv_silu(rows, col0, channels, weight, bias, history, ctx) -> torch.Tensor:
+    """silu of a causal convolution per channel over ``channels`` columns of the float32 ``rows`` from ``col0`` on;
+    weight float32 [channels, taps] (last column: the current token), bias [channels] or None; ``history``
+    float32 [slots, taps - 1, channels] holds every sequence's last inputs and is brought up to date."""
+    _dev(rows, weight, bias, history)
+    _f32_rows(rows, "conv rows")
+    t, taps = rows.shape[0], weight.shape[1]
+    _need(weight.dtype == torch.float32 and weight.shape == (channels, taps) and 1 <= taps <= 16, "conv weight: float32 [channels, taps <= 16]")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.shape == (channels,)), "conv bias: float32 [channels]")
+    _need(0 <= col0 and col0 + channels <= rows.shape[1], "conv: columns beyond the rows")
+    _need(history.dtype == torch.float32 and history.dim() == 3 and tuple(history.shape[1:]) == (max(taps - 1, 1), channels),
+          "conv history: float32 [slots, taps - 1, channels]")
+    _i32(ctx.pos, t, "positions")
+    _i32(ctx.tok_slot, t, "slots")
+    _i32(ctx.seq_slot, ctx.n_seqs, "sequence slots")
+    qstart, qlen = getattr(ctx, "seq_qstart", None), getattr(ctx, "seq_qlen", None)
+    _need((qstart is None) == (qlen is None) and (qstart is not None or t == ctx.n_seqs), "conv: per-sequence starts and lengths")
+    out = torch.empty((t, channels), dtype=torch.float32, device=rows.device)
+    _check(hybrid().li_conv_silu(_ptr(rows), rows.shape[1], col0, _ptr(weight), _ptr(bias), _ptr(history), _ptr(ctx.pos),
+                                 _ptr(ctx.tok_slot), _ptr(ctx.seq_slot), _ptr(qstart), _ptr(qlen), _ptr(out), t, ctx.n_seqs,
+                                 channels, taps, _stream()), "conv_silu")
+    return out
+
+
+def ssm_scan(xbc, proj, dt_col, dt_bias, a_log, d_skip, state, ctx, heads, groups, n_state, dv) -> torch.Tensor:
+    """The selective state-space recurrence, token by token in float32.  ``xbc`` float32 [T, heads * dv + 2 groups
+    n_state] (x | B | C), the raw step sizes in ``proj`` columns dt_col .. dt_col + heads; ``state`` float32
+    [slots, heads, n_state, dv], read and left up to date; returns y float32 [T, heads * dv]."""
+    _dev(xbc, proj, dt_bias, a_log, d_skip, state)
+    _f32_rows(xbc, "ssm x/B/C")
+    _f32_rows(proj, "ssm projections")
+    t = xbc.shape[0]
+    _need(heads % groups == 0 and n_state <= 256, "ssm: heads a multiple of groups, a state of up to 256")
+    _need(xbc.shape[1] == heads * dv + 2 * groups * n_state and proj.shape[0] == t and dt_col + heads <= proj.shape[1], "ssm: row widths")
+    for v in (dt_bias, a_log, d_skip):
+        _need(v is None or (v.dtype == torch.float32 and v.shape == (heads,)), "ssm: float32 [heads] vectors")
+    _need(dt_bias is not None and a_log is not None, "ssm: dt_bias and A_log")
+    _need(state.dtype == torch.float32 and tuple(state.shape[1:]) == (heads, n_state, dv), "ssm state: float32 [slots, heads, N, dv]")
+    _i32(ctx.seq_slot, ctx.n_seqs, "sequence slots")
+    qstart, qlen = getattr(ctx, "seq_qstart", None), getattr(ctx, "seq_qlen", None)
+    _need((qstart is None) == (qlen is None) and (qstart is not None or t == ctx.n_seqs), "ssm: per-sequence starts and lengths")
+    y = torch.empty((t, heads * dv), dtype=torch.float32, device=xbc.device)
+    _check(hybrid().li_ssm_scan(_ptr(xbc), xbc.shape[1], _ptr(proj), proj.shape[1], dt_col, _ptr(dt_bias), _ptr(a_log),
+                                _ptr(d_skip), _ptr(state), _ptr(ctx.seq_slot), _ptr(qstart), _ptr(qlen), _ptr(y), ctx.n_seqs,
+                                heads, groups, n_state, dv, _stream()), "ssm_scan")
+    return y
+
+
+def gated_group_norm(y, zrows, z_col, weight, groups, eps, out_dtype) -> torch.Tensor:
+    """(y * silu(z)) divided, in ``groups`` equal parts of a row, by each part's root mean square, times weight."""
+    _dev(y, zrows, weight)
+    _f32_rows(y, "gated norm y")
+    _f32_rows(zrows, "gated norm z")
+    t, n = y.shape
+    _need(n % groups == 0 and zrows.shape[0] == t and 0 <= z_col and z_col + n <= zrows.shape[1], "gated norm: sizes")
+    _need(weight.dtype == torch.float32 and weight.shape == (n,), "gated norm weight: float32 [n]")
+    out = torch.empty((t, n), dtype=out_dtype, device=y.device)
+    _check(hybrid().li_gated_group_norm(_ptr(y), _ptr(zrows), zrows.shape[1], z_col, _ptr(weight), _ptr(out), DT[out_dtype],
+                                        t, n, groups, c_float(eps), _stream()), "gated_group_norm")
+    return out
+
+
+def moe_route(logits, correction, h, residual, n_route, n_real, top, has_gate, scale) -> torch.Tensor:
+    """Routing weights of every token: softmax over the first ``n_route`` columns of ``logits`` (float32), the ``top``
+    largest of score + correction chosen, their scores divided by their sum (+ 1e-20) times ``scale``.  Returns
+    float32 [T, n_real (+ 1)]: the weights of the first ``n_real`` outputs (0 where not chosen) and, with
+    ``has_gate`` 1, sigmoid of the column behind the router's (2: the constant 1; 0: no such column).  The outputs from ``n_real`` on pass the token on:
+    residual[t] += (their weights' sum) * h[t]."""
+    _dev(logits, correction, h, residual)
+    _f32_rows(logits, "router logits")
+    t, width = h.shape
+    has_gate = int(has_gate)
+    _need(logits.shape[0] == t and logits.shape[1] >= n_route + int(has_gate == 1), "router logits: a row for every token")
+    _need(1 <= top <= n_route and 0 <= n_real <= n_route, "router: top within the outputs")
+    _need(correction is None or (correction.dtype == torch.float32 and correction.shape == (n_route,)), "router correction: float32 [outputs]")
+    _need(h.dtype in DT and residual.dtype == torch.float32 and residual.shape == h.shape, "router: h and the float32 residual rows")
+    _drop_row_stats(residual)
+    w = torch.empty((t, n_real + int(bool(has_gate))), dtype=torch.float32, device=h.device)
+    _check(hybrid().li_moe_route(_ptr(logits), logits.shape[1], _ptr(correction), _ptr(h), DT[h.dtype], _ptr(residual), _ptr(w),
+                                 t, width, n_route, n_real, top, has_gate, c_float(scale), _stream()), "moe_route")
+    return w
+
+
+def scale_blocks(t, weights, n_blocks, ff, tail) -> torch.Tensor:
+    """In place: block e (``ff`` columns) of every row of ``t`` times weights[row][e]; the last ``tail`` columns
+    times weights[row][n_blocks]."""
+    _dev(t, weights)
+    _need(t.dim() == 2 and t.dtype in DT and t.shape[1] == n_blocks * ff + tail, "scale_blocks: [T, blocks * ff + tail]")
+    _need(weights.dtype == torch.float32 and weights.shape == (t.shape[0], n_blocks + int(tail > 0)), "scale_blocks: a weight for every block")
+    _check(hybrid().li_scale_blocks(_ptr(t), DT[t.dtype], _ptr(weights), t.shape[0], n_blocks, ff, tail, _stream()), "scale_blocks")
+    return t
+
+
+def copy_rows(x: torch.Tensor) -> torch.Tensor:
+    """A copy of ``x`` in memory of its own (one device-to-device copy on the current stream)."""
+    return x.clone()

@@ -2,14 +2,18 @@ from .base import Part, collect_params
 from .norm import LayerNorm, RMSNorm
 from .position import RotaryPosition, NoPosition
 from .attention import Attention
-from .feed_forward import GatedMLP, PolyNormMLP
+from .feed_forward import DenseMLP, GatedMLP, PolyNormMLP, RoutedExperts
 from .token_shift import ShiftedMixer
 from .parallel import ParallelMixers
 from .sigmoid_attention import SigmoidAttention
 from .decay_attention import DecayLinearAttention
+from .diff_attention import DifferentialAttention
+from .state_space import SelectiveStateSpace
+from .stream import Reinject
 from .embedding import Embedding, LMHead
 from .block import Block, PostNormBlock, PreNormBlock, SubLayer
 
 __all__ = ["Part", "collect_params", "RMSNorm", "RotaryPosition", "NoPosition", "Attention", "GatedMLP",
            "Embedding", "LMHead", "Block", "PreNormBlock", "SubLayer", "LayerNorm", "PolyNormMLP", "ShiftedMixer",
-           "ParallelMixers", "SigmoidAttention", "DecayLinearAttention", "PostNormBlock"]
+           "ParallelMixers", "SigmoidAttention", "DecayLinearAttention", "PostNormBlock", "DifferentialAttention",
+           "SelectiveStateSpace", "Reinject", "DenseMLP", "RoutedExperts"]

@@ -10,12 +10,22 @@ from .base import Part
 
 @register_embedding("embedding")
 class Embedding(Part):
-    """x = float32(table[token]), unscaled (src/model/model.cpp:101-118)."""
+    """x = float32(table[token]) (src/model/model.cpp:101-118), times ``scale``; ``positions`` "sinusoidal" adds
+    to every token the vector of its position p: entry 2i is sin(p f_i), entry 2i+1 cos(p f_i), with
+    f_i = position_base^(-2i / hidden_size) (float32 angles)."""
 
-    def __init__(self, *, vocab_size, hidden_size, name="weight", prefix, dtype, device):
+    def __init__(self, *, vocab_size, hidden_size, name="weight", scale=1.0, positions=None, position_base=10000.0,
+                 prefix, dtype, device):
+        if positions not in (None, "sinusoidal"):
+            raise ValueError(f"embedding: positions {positions!r} are not built ('sinusoidal' is)")
         self.vocab_size, self.hidden_size, self.name = vocab_size, hidden_size, name
+        self.scale, self.positions = float(scale), positions
         self.prefix, self.dtype, self.device = prefix, dtype, device
-        self.weight = None
+        self.weight = self.freq = None
+        if positions is not None:
+            two_i = torch.arange(0, hidden_size, 2, dtype=torch.float64)
+            self.freq = torch.pow(torch.tensor(float(position_base), dtype=torch.float64), -two_i / hidden_size) \
+                .to(torch.float32).to(device or "cpu")
 
     def params(self):
         return {self.name: ParamSpec((self.vocab_size, self.hidden_size))}
@@ -26,7 +36,9 @@ class Embedding(Part):
     def forward(self, ctx):
         """The residual stream's first value for the step's tokens, float32 [T, hidden].  ``ctx`` is the
         step (``token_ids``, and ``pos`` for an embedding that adds positions)."""
-        return ops.embed(self.weight, ctx.token_ids)
+        if self.positions is None and self.scale == 1.0:
+            return ops.embed(self.weight, ctx.token_ids)
+        return ops.embed_positions(self.weight, ctx.token_ids, ctx.pos, self.freq, self.scale)
 
 
 @register_head("lm_head")
@@ -34,20 +46,20 @@ class LMHead(Part):
     """logits = h W^T in float32 (src/model/model.cpp:93-98).  ``tied``: W is the embedding
     table (the reference has no tied models: it requires output.weight, model.cpp:35-38)."""
 
-    def __init__(self, *, vocab_size, hidden_size, tied, prefix, dtype, device):
-        self.vocab_size, self.hidden_size, self.tied = vocab_size, hidden_size, tied
+    def __init__(self, *, vocab_size, hidden_size, tied, name="weight", prefix, dtype, device):
+        self.vocab_size, self.hidden_size, self.tied, self.name = vocab_size, hidden_size, tied, name
         self.prefix, self.dtype, self.device = prefix, dtype, device
         self.weight = None
 
     def params(self):
-        return {} if self.tied else {"weight": ParamSpec((self.vocab_size, self.hidden_size))}
+        return {} if self.tied else {self.name: ParamSpec((self.vocab_size, self.hidden_size))}
 
     def ignorable(self):
-        return [self.prefix + "weight"] if self.tied else []
+        return [self.prefix + self.name] if self.tied else []
 
     def bind(self, tensors):
         if not self.tied:
-            self.weight = ops.prepare_weight(tensors["weight"])
+            self.weight = ops.prepare_weight(tensors[self.name])
 
     def tie(self, table):
         # the embedding gathers rows, the head streams the whole matrix: it keeps a tiled copy

@@ -76,3 +76,100 @@ class PolyNormMLP(Part):
     def forward(self, h, residual):
         ops.linear(ops.polynorm(ops.linear(h, self.w_up, out_dtype=torch.float32), self.coef, self.eps, self.dtype),
                    self.w_down, ops.EPI_ADD, out=residual)
+
+
+@register_feed_forward("dense_mlp")
+class DenseMLP(Part):
+    """down(act(up(x))) added into the residual stream: no gate.  ``activation``: "gelu" (the exact form with
+    erf), "gelu_tanh" or "silu", computed in float32 on the product's sums.  ``names``: local tensor names."""
+
+    takes_lazy_norm = True
+
+    def __init__(self, *, hidden_size, intermediate_size, activation="gelu", names=None, prefix, dtype, device):
+        if activation not in ops.ACTIVATIONS:
+            raise ValueError(f"dense_mlp: activation {activation!r} is not built ({', '.join(ops.ACTIVATIONS)} are)")
+        self.hidden_size, self.intermediate_size, self.activation = hidden_size, intermediate_size, activation
+        self.names = {"up": "up_proj.weight", "down": "down_proj.weight", **(names or {})}
+        self.prefix, self.dtype, self.device = prefix, dtype, device
+        self.w_up = self.w_down = None
+
+    def params(self):
+        f, d, n = self.intermediate_size, self.hidden_size, self.names
+        return {n["up"]: ParamSpec((f, d)), n["down"]: ParamSpec((d, f))}
+
+    def bind(self, tensors):
+        n = self.names
+        self.w_up, self.w_down = ops.prepare_weight(tensors[n["up"]]), ops.prepare_weight(tensors[n["down"]])
+
+    def forward(self, h, residual):
+        z = ops.linear(h, self.w_up, out_dtype=torch.float32)
+        ops.linear(ops.activation(z, self.activation, self.dtype), self.w_down, ops.EPI_ADD, out=residual)
+
+
+@register_feed_forward("routed_experts")
+class RoutedExperts(Part):
+    """A mixture of ``n_experts`` gated feed-forwards down(silu(gate(h)) * up(h)) of width ``expert_ff`` (tensors
+    ``e<i>.gate``, ``e<i>.up``, ``e<i>.down``), of which every token uses ``top``.
+
+    The router has n_experts + ``n_identity`` outputs; its logits and everything after them are float32:
+    s = softmax(W_router h); the ``top`` outputs with the largest s + correction are chosen (``correction``: a
+    tensor with one number an output, used for the choice only); their weights are s / (sum of the chosen s +
+    1e-20) * ``route_scale``.  The last ``n_identity`` outputs have no matrices: chosen, they add weight * h.
+    ``shared_ff`` > 0: one more expert of that width runs for every token; ``shared_gate``: it is weighted by
+    sigmoid(w_sg . h).
+
+    How it runs: the experts' gate and up matrices are stacked (the shared expert's behind them) into one
+    product whose epilogue applies silu(gate) * up; every expert's block of the hidden row is multiplied by the
+    token's weight for that expert, zero where it was not chosen; one product against the down matrices side by
+    side then sums the experts.  Every token so runs through every expert's matrices: the same numbers as
+    running only the chosen ones, no sorting of tokens, no shapes that depend on the data (a step can be
+    recorded), at n_experts / top times the arithmetic."""
+
+    def __init__(self, *, hidden_size, n_experts, expert_ff, top, n_identity=0, route_scale=1.0, correction=True,
+                 shared_ff=0, shared_gate=True, names=None, prefix, dtype, device):
+        if not 1 <= top <= n_experts + n_identity:
+            raise ValueError(f"routed experts: top {top} of {n_experts + n_identity} outputs")
+        self.hidden_size, self.n_experts, self.expert_ff, self.top = hidden_size, n_experts, expert_ff, top
+        self.n_identity, self.route_scale, self.correction = n_identity, float(route_scale), bool(correction)
+        self.shared_ff, self.shared_gate = int(shared_ff or 0), bool(shared_gate) and bool(shared_ff)
+        self.names = {"router": "router.weight", "correction": "router.correction", "expert": "e{}.", "shared": "shared.",
+                      "gate": "gate", "up": "up", "down": "down", "shared_gate": "shared.sg", **(names or {})}
+        self.prefix, self.dtype, self.device = prefix, dtype, device
+        self.w_router = self.w_gate_up = self.w_down = self.bias = None
+
+    def _experts(self):
+        n = self.names
+        out = [(n["expert"].format(i), self.expert_ff) for i in range(self.n_experts)]
+        return out + ([(n["shared"], self.shared_ff)] if self.shared_ff else [])
+
+    def params(self):
+        n, d = self.names, self.hidden_size
+        out = {n["router"]: ParamSpec((self.n_experts + self.n_identity, d), "vector", "wide")}
+        if self.correction:
+            out[n["correction"]] = ParamSpec((self.n_experts + self.n_identity,), "vector", "small")
+        for p, f in self._experts():
+            out.update({p + n["gate"]: ParamSpec((f, d)), p + n["up"]: ParamSpec((f, d)), p + n["down"]: ParamSpec((d, f))})
+        if self.shared_gate:
+            out[n["shared_gate"]] = ParamSpec((1, d), "vector", "wide")
+        return out
+
+    def bind(self, tensors):
+        n, d = self.names, self.hidden_size
+        gu, down = [], []
+        for p, f in self._experts():
+            g, u = tensors[p + n["gate"]], tensors[p + n["up"]]
+            gu.append(torch.stack([g, u], dim=1).reshape(2 * f, d))            # row 2j: gate_j, row 2j + 1: up_j
+            down.append(tensors[p + n["down"]])
+        self.w_gate_up = ops.prepare_weight(torch.cat(gu, 0).contiguous())
+        self.w_down = ops.prepare_weight(torch.cat(down, 1).contiguous())
+        rows = [tensors[n["router"]].float()] + ([tensors[n["shared_gate"]].float().view(1, d)] if self.shared_gate else [])
+        self.w_router = ops.prepare_weight(torch.cat(rows, 0).contiguous())   # float32: the logits are summed in float32
+        self.bias = tensors[n["correction"]] if self.correction else None
+
+    def forward(self, h, residual):
+        logits = ops.linear(h, self.w_router, out_dtype=torch.float32)
+        weights = ops.moe_route(logits, self.bias, h, residual, self.n_experts + self.n_identity, self.n_experts, self.top,
+                                (1 if self.shared_gate else 2) if self.shared_ff else 0, self.route_scale)
+        t = ops.linear(h, self.w_gate_up, ops.EPI_SWIGLU, out_dtype=self.dtype)
+        ops.scale_blocks(t, weights, self.n_experts, self.expert_ff, self.shared_ff)
+        ops.linear(t, self.w_down, ops.EPI_ADD, out=residual)

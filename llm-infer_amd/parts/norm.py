@@ -4,6 +4,7 @@ import torch
 
 from ..kernels import ops
 from ..registry import register_norm
+from ..tensor import Tensor
 from ..weights.loader import ParamSpec
 from .base import Part
 
@@ -14,15 +15,19 @@ class RMSNorm(Part):
     (include/kernels_cpu.hpp:43-54, src/model/block.cpp:81-83)."""
     can_be_lazy = True          # forward takes ``lazy``
 
-    def __init__(self, *, size: int, eps: float, prefix: str, dtype, device):
+    def __init__(self, *, size: int, eps: float, name: str = "weight", one_plus: bool = False, prefix: str, dtype, device):
+        """``name``: local name of the weight's tensor.  ``one_plus``: the tensor is stored around zero and the
+        rows are multiplied by 1 + w (added once, in float32, when the weights are bound)."""
         self.size, self.eps, self.prefix, self.dtype, self.device = size, float(eps), prefix, dtype, device
+        self.name, self.one_plus = name, bool(one_plus)
         self.weight = None
 
     def params(self):
-        return {"weight": ParamSpec((self.size,), "vector", "ones")}
+        return {self.name: ParamSpec((self.size,), "vector", "small" if self.one_plus else "ones")}
 
     def bind(self, tensors):
-        self.weight = tensors["weight"]
+        w = tensors[self.name]
+        self.weight = Tensor.wrap((w.as_subclass(torch.Tensor).float() + 1.0).contiguous()) if self.one_plus else w
 
     def forward(self, x: torch.Tensor, rows: torch.Tensor | None = None, lazy: bool = False):
         """The normed rows in the compute dtype.  ``lazy``: the caller hands the result to parts that pass

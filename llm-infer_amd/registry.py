@@ -24,9 +24,10 @@ POSITIONS: dict = {}
 BLOCKS: dict = {}
 EMBEDDINGS: dict = {}
 HEADS: dict = {}
+STREAMS: dict = {}
 
 _TABLES = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS, "position": POSITIONS,
-           "block": BLOCKS, "embedding": EMBEDDINGS, "head": HEADS}
+           "block": BLOCKS, "embedding": EMBEDDINGS, "head": HEADS, "stream": STREAMS}
 
 
 def register_architecture(name: str, config_cls) -> None:
@@ -47,6 +48,7 @@ def register_position(kind): return _register("position", kind)
 def register_block(kind): return _register("block", kind)
 def register_embedding(kind): return _register("embedding", kind)
 def register_head(kind): return _register("head", kind)
+def register_stream(kind): return _register("stream", kind)
 
 
 def lookup(table_name: str, kind: str):

@@ -1,7 +1,8 @@
 """Random-weights mode: tensors from a parameter table and a seed.
 
 Matrices and tables are N(0, 0.02), norm vectors 1 + N(0, 0.01); a vector whose ``init`` is "small" is
-N(0, 0.02) (a bias), one whose ``init`` is "half" 0.5 + N(0, 0.1) within [0, 1] (mixing weights).  Every tensor
+N(0, 0.02) (a bias), one whose ``init`` is "half" 0.5 + N(0, 0.1) within [0, 1] (mixing weights), one whose ``init``
+is "wide" N(0, 0.4) (a short convolution).  Every tensor
 has a generator of its own, seeded by (seed, tensor name), so a tensor's values
 depend on neither the order nor the presence of the others.  The reference has
 no such mode.
@@ -31,6 +32,8 @@ def random_tensor(name: str, spec, seed: int, matrix_dtype: torch.dtype, device=
         raise ValueError(f"{name}: integer tables have no random initialisation")
     if spec.init == "small":         # a bias or another vector around zero
         return MATRIX_STD * torch.randn(spec.shape, generator=g, device=device, dtype=torch.float32)
+    if spec.init == "wide":          # weights of a short convolution and the like: of the order of one half
+        return 0.4 * torch.randn(spec.shape, generator=g, device=device, dtype=torch.float32)
     if spec.init == "half":          # mixing weights between 0 and 1
         return (0.5 + 0.1 * torch.randn(spec.shape, generator=g, device=device, dtype=torch.float32)).clamp_(0.0, 1.0)
     if spec.kind == "vector" or spec.init == "ones":
