@@ -62,7 +62,7 @@ def main() -> int:
                     help="leave out the long contexts, batch 128 and the generation run that the default run adds to points")
     ap.add_argument("--generate", type=int, default=0,
                     help="also generate for this many 128-token prompts with budgets drawn from 16..512 tokens")
-    ap.add_argument("--compare", default="", choices=["", "manirax"],
+    ap.add_argument("--compare", default="", choices=["", "manirax", "risonex"],
                     help="instead of the default workload: prefill and decode throughput of this design at a few "
                          "layer sizes beside the Llama decoder at equal sizes (random weights, a few layers each)")
     ap.add_argument("--sizes", default="", help="with --compare: the layer sizes to run, comma separated (default: all)")
@@ -147,6 +147,22 @@ def compare_configs(design: str, size: dict, layers: int, context: int) -> dict:
                  num_key_value_heads=G, head_dim=hd, intermediate_size=size["ff"], vocab_size=size["vocab"],
                  rope_theta=500000.0, rms_norm_eps=1e-5, max_position_embeddings=context, tie_word_embeddings=True,
                  hidden_act="silu")
+    if design == "risonex":
+        # state-space layers (twice the width inside, 64 values a head, a state of 128) alternating with differential
+        # attention of the same heads (two maps of half a head each, values a head wide, blocks of 1,024 positions); a
+        # dense feed-forward of the Llama decoder's width in the first layer, then eight experts of a quarter of
+        # it, two of them chosen, beside a shared one
+        ssm = {"type": "mamba2", "mixer": {"heads": 2 * w // 64, "vdim": 64, "state": 128, "groups": 1, "conv": 4,
+                                           "norm_groups": 1}}
+        att = {"type": "attention", "mixer": {"heads": H, "kv_heads": G, "dim": hd // 2, "vdim": hd, "diff": 0.3,
+                                              "scale": (hd // 2) ** -0.5, "mask": {"size": 1024}}}
+        routed = {"kind": "moe", "expert": {"ff": size["ff"] // 4}, "shared": {"ff": size["ff"] // 4},
+                  "router": {"experts": 8, "identity": 0, "top": 2, "scale": 1.0}}
+        stack = [dict(ssm if i % 2 == 0 else att, mlp={"kind": "dense", "ff": size["ff"]} if i == 0 else routed)
+                 for i in range(layers)]
+        other = {"architecture": "Risonex", "embedding": {"scale": 1.0}, "layers": stack, "norm": {"eps": 1e-5},
+                 "vocab": size["vocab"], "width": w, "max_positions": context}
+        return {"llama": llama, design: other}
     assert design == "manirax"
     # the attention of the same heads beside a linear attention of half as many heads with states of hd x hd
     layer = {"type": "parallel", "mlp": {"kind": "dense", "ff": size["ff"]},

@@ -59,27 +59,36 @@ def chunk_mask(n, size):
     return (j <= i) & (i // size == j // size)
 
 
-def diff_attention(h, t, m, eps):
-    """``t``: the mixer's tensors by local name (q, k, v, o, q.norm, k.norm, lq1, lk1, lq2, lk2); ``m``: its sizes."""
-    H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    n = h.shape[0]
-    q = (h @ t["q"].T).view(n, H, 2, d)
-    k = (h @ t["k"].T).view(n, G, 2, d)
-    v = (h @ t["v"].T).view(n, G, dv)
-    q = rms_div(q, eps) * t["q.norm"]
-    k = rms_div(k, eps) * t["k.norm"]
-    lam = torch.exp((t["lq1"] * t["lk1"]).sum()) - torch.exp((t["lq2"] * t["lk2"]).sum()) + m["diff"]
-    see = chunk_mask(n, int(m["mask"]["size"]))
-    out = torch.zeros((n, H, dv), dtype=h.dtype)
+def diff_attention_core(q, k, v, scale, lam, size, eps, out_scale):
+    """q [n, H, 2, d], k [n, G, 2, d], v [n, G, dv] -> [n, H, dv]: two softmax maps over the same values, their
+    difference divided by its root mean square (``eps`` None: left as it is) and multiplied by ``out_scale``."""
+    n, H, G = q.shape[0], q.shape[1], k.shape[1]
+    see = chunk_mask(n, size)
+    out = torch.zeros((n, H, v.shape[-1]), dtype=q.dtype)
     for head in range(H):
         g = head // (H // G)
         maps = []
         for which in range(2):
-            s = (q[:, head, which] @ k[:, g, which].T) * m["scale"]
+            s = (q[:, head, which] @ k[:, g, which].T) * scale
             s = s.masked_fill(~see, float("-inf"))
             maps.append(torch.softmax(s, dim=-1) @ v[:, g])
         o = maps[0] - lam * maps[1]
-        out[:, head] = rms_div(o, eps) * (1.0 - m["diff"])
+        out[:, head] = (o if eps is None else rms_div(o, eps)) * out_scale
+    return out
+
+
+def diff_lambda(t, diff):
+    return torch.exp((t["lq1"] * t["lk1"]).sum()) - torch.exp((t["lq2"] * t["lk2"]).sum()) + diff
+
+
+def diff_attention(h, t, m, eps):
+    """``t``: the mixer's tensors by local name (q, k, v, o, q.norm, k.norm, lq1, lk1, lq2, lk2); ``m``: its sizes."""
+    H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+    n = h.shape[0]
+    q = rms_div((h @ t["q"].T).view(n, H, 2, d), eps) * t["q.norm"]
+    k = rms_div((h @ t["k"].T).view(n, G, 2, d), eps) * t["k.norm"]
+    v = (h @ t["v"].T).view(n, G, dv)
+    out = diff_attention_core(q, k, v, m["scale"], diff_lambda(t, m["diff"]), int(m["mask"]["size"]), eps, 1.0 - m["diff"])
     return out.reshape(n, H * dv) @ t["o"].T
 
 
