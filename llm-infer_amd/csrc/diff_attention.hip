@@ -1,0 +1,205 @@
+// Differential attention over blocks of positions on the matrix cores, for one pair of sizes: MAP_DIM (a map's
+// key size rounded up to 16) and VALUE_DIM (the value size rounded up to 32), both compile-time.  16-bit keys,
+// values and queries; scores, weights, sums and the norm of the output float32.
+//
+// One wave per (tile of up to 32 consecutive tokens of a sequence, query head); a decode step's tiles hold one
+// token.  A token at position p sees the keys lo .. p, lo = p - p % block (block 0: 0; window w: at least p - w + 1).
+// Keys are walked 32 at a time.  Per map m:  S^T = K_m Q_m^T  (rows keys, columns queries; operand A straight from
+// the page, which holds keys in operand order), online softmax down the rows (a query's 32 scores lie in the 16
+// accumulator elements of two lanes), then O_m^T += V^T P_m^T with the accumulators' own order of the keys, in which the
+// page holds the values.  A weight enters the second product as the sum of two 16-bit numbers (its rounding and the
+// rounding of the remainder), so that the product sees 16 bits of it.  At the end o = O_1 / l_1 - lambda O_2 / l_2,
+// divided by its root mean square over the value size and multiplied by out_scale.
+#include "common.h"
+
+#ifndef MAP_DIM
+#error "compile with -DMAP_DIM=<multiple of 16> -DVALUE_DIM=<multiple of 32>"
+#endif
+static_assert(MAP_DIM % 16 == 0 && MAP_DIM >= 16 && MAP_DIM <= 256, "a map's key size: a multiple of 16 up to 256");
+static_assert(VALUE_DIM % 32 == 0 && VALUE_DIM >= 32 && VALUE_DIM <= 256, "value size: a multiple of 32 up to 256");
+
+struct MapPages {
+    const void* k;
+    const void* v;
+    int64_t page_stride;
+    const int* page_table;
+    int max_pages;
+};
+
+template <class T, int MAPS>
+__global__ __launch_bounds__(64) void diff_attn_mfma_kernel(
+    const T* __restrict__ q, T* __restrict__ out, MapPages pg, const int* __restrict__ pos,
+    const int* __restrict__ tok_slot, const int* __restrict__ tile_t0, const int* __restrict__ tile_n, int H, int G,
+    int dv, float scale, int block, int window, float lambda, float out_eps, float out_scale) {
+    typedef typename Vec<T>::v8 v8;
+    constexpr int D16 = MAP_DIM / 16, KW = MAPS * MAP_DIM, DVB = VALUE_DIM / 32;
+    const int tile = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, col = lane & 31, half = lane >> 5;
+    const int t0 = tile_t0 ? tile_t0[tile] : tile, n = tile_n ? tile_n[tile] : 1;
+    if (n <= 0) return;
+    const int g = h / (H / G);
+    const int p0 = pos[t0];                            // the tile's tokens stand at p0, p0 + 1, ...
+    const bool has_query = col < n;
+    const int pq = p0 + min(col, n - 1);
+    int lo_q = block > 0 ? pq - pq % block : 0;
+    if (window > 0) lo_q = max(lo_q, pq - window + 1);
+    int lo_tile = block > 0 ? p0 - p0 % block : 0;     // the first token's: the smallest
+    if (window > 0) lo_tile = max(lo_tile, p0 - window + 1);
+    const int p_last = p0 + n - 1;
+    const int* table = pg.page_table + (int64_t)tok_slot[t0] * pg.max_pages;
+
+    v8 qf[MAPS][D16];
+    {
+        const T* qrow = q + ((int64_t)(t0 + min(col, n - 1)) * H + h) * KW;
+#pragma unroll
+        for (int a = 0; a < MAPS; ++a)
+#pragma unroll
+            for (int s = 0; s < D16; ++s) qf[a][s] = *(const v8*)(qrow + a * MAP_DIM + s * 16 + half * 8);
+    }
+    f32x16 o[MAPS][DVB];
+    float m[MAPS], l[MAPS];
+#pragma unroll
+    for (int a = 0; a < MAPS; ++a) {
+        m[a] = -INFINITY; l[a] = 0.f;
+#pragma unroll
+        for (int b = 0; b < DVB; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[a][b][r] = 0.f;
+    }
+
+    // the fragments of the 32 keys after the ones at work are fetched before the work begins
+    v8 kn[MAPS][D16], vn[DVB][2];
+    auto fetch = [&](int kt) {
+        const int page = table[kt >> 1], tb = kt & 1;                      // two blocks of 32 keys a page
+        const T* kh = (const T*)pg.k + (int64_t)page * pg.page_stride + g * k_head_elems(KW);
+        const T* vh = (const T*)pg.v + (int64_t)page * pg.page_stride + g * v_head_elems(VALUE_DIM);
+#pragma unroll
+        for (int a = 0; a < MAPS; ++a)
+#pragma unroll
+            for (int s = 0; s < D16; ++s) kn[a][s] = *(const v8*)(kh + ((int64_t)(tb * (KW / 16) + a * D16 + s) * 64 + lane) * 8);
+#pragma unroll
+        for (int b = 0; b < DVB; ++b)
+#pragma unroll
+            for (int u = 0; u < 2; ++u) vn[b][u] = *(const v8*)(vh + ((int64_t)(b * (PAGE / 16) + tb * 2 + u) * 64 + lane) * 8);
+    };
+    const int kt_last = p_last / 32;
+    fetch(lo_tile / 32);
+    for (int kt = lo_tile / 32; kt <= kt_last; ++kt) {
+        v8 kf[MAPS][D16], vf[DVB][2];
+#pragma unroll
+        for (int a = 0; a < MAPS; ++a)
+#pragma unroll
+            for (int s = 0; s < D16; ++s) kf[a][s] = kn[a][s];
+#pragma unroll
+        for (int b = 0; b < DVB; ++b)
+#pragma unroll
+            for (int u = 0; u < 2; ++u) vf[b][u] = vn[b][u];
+        if (kt < kt_last) fetch(kt + 1);
+        v8 phi[MAPS][2], plo[MAPS][2];
+#pragma unroll
+        for (int a = 0; a < MAPS; ++a) {
+            f32x16 acc;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+            for (int s = 0; s < D16; ++s) {
+                acc = mfma32(kf[a][s], qf[a][s], acc);
+            }
+            float tmax = -INFINITY;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int key = kt * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+                const bool seen = has_query && key >= lo_q && key <= pq;
+                acc[r] = seen ? acc[r] * scale : -INFINITY;
+                tmax = fmaxf(tmax, acc[r]);
+            }
+            tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
+            const float mn = fmaxf(m[a], tmax);
+            float f = 1.f, sum = 0.f;
+            float pr[16];
+            if (mn == -INFINITY) {                                         // nothing seen yet by this query
+#pragma unroll
+                for (int r = 0; r < 16; ++r) pr[r] = 0.f;
+            } else {
+                f = expf(m[a] - mn);                                       // 0 while m is still -inf
+#pragma unroll
+                for (int r = 0; r < 16; ++r) { pr[r] = expf(acc[r] - mn); sum += pr[r]; }
+            }
+            sum += __shfl_xor(sum, 32, WAVE);
+            l[a] = l[a] * f + sum;
+            m[a] = mn;
+            if (f != 1.f) {
+#pragma unroll
+                for (int b = 0; b < DVB; ++b)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) o[a][b][r] *= f;
+            }
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const T hi = from_f32<T>(pr[8 * u + i]);
+                    phi[a][u][i] = hi;
+                    plo[a][u][i] = from_f32<T>(pr[8 * u + i] - to_f32(hi));
+                }
+        }
+#pragma unroll
+        for (int b = 0; b < DVB; ++b)
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+#pragma unroll
+                for (int a = 0; a < MAPS; ++a) {
+                    o[a][b] = mfma32(vf[b][u], phi[a][u], o[a][b]);
+                    o[a][b] = mfma32(vf[b][u], plo[a][u], o[a][b]);
+                }
+            }
+    }
+    // o = O_1 / l_1 - lambda O_2 / l_2 for this lane's query; its values lie in this lane and in lane ^ 32
+    float ss = 0.f;
+#pragma unroll
+    for (int b = 0; b < DVB; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int dim = b * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+            float v = o[0][b][r] / l[0];
+            if (MAPS == 2) v -= lambda * (o[MAPS - 1][b][r] / l[MAPS - 1]);
+            v = dim < dv ? v : 0.f;
+            o[0][b][r] = v;
+            ss += v * v;
+        }
+    ss += __shfl_xor(ss, 32, WAVE);
+    const float rr = out_eps >= 0.f ? out_scale / sqrtf(ss / (float)dv + out_eps) : out_scale;
+    if (has_query) {
+        T* orow = out + ((int64_t)(t0 + col) * H + h) * dv;
+#pragma unroll
+        for (int b = 0; b < DVB; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int dim = b * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+                if (dim < dv) orow[dim] = from_f32<T>(o[0][b][r] * rr);
+            }
+    }
+}
+
+extern "C" int li_diffattn_map_dim() { return MAP_DIM; }
+extern "C" int li_diffattn_value_dim() { return VALUE_DIM; }
+
+// q [T, H, maps * MAP_DIM] and out [T, H * dv] of type dt (float16 or bfloat16), as are the pages.  tile_t0 / tile_n
+// (device, may be null: every token a tile of its own): first row and number of rows (1 .. 32) of every tile.
+extern "C" int li_diffattn(const void* q, void* out, int dt, const void* k_pages, const void* v_pages, int64_t page_stride,
+                           const int* page_table, int max_pages, const int* pos, const int* tok_slot, const int* tile_t0,
+                           const int* tile_n, int n_tiles, int H, int G, int maps, int dv, float scale, int block, int window,
+                           float lambda, float out_eps, float out_scale, hipStream_t stream) {
+    if (n_tiles <= 0) return LI_OK;
+    if (H <= 0 || G <= 0 || H % G || dv <= 0 || dv > VALUE_DIM || block < 0 || window < 0) return LI_BAD_ARG;
+    if (maps < 1 || maps > 2 || (dt != DT_F16 && dt != DT_BF16)) return LI_UNSUPPORTED;
+    if ((tile_t0 == nullptr) != (tile_n == nullptr)) return LI_BAD_ARG;
+    MapPages pg{k_pages, v_pages, page_stride, page_table, max_pages};
+    dim3 grid(n_tiles, H);
+#define GO(T, M) diff_attn_mfma_kernel<T, M><<<grid, 64, 0, stream>>>((const T*)q, (T*)out, pg, pos, tok_slot, tile_t0, tile_n, \
+                                                                      H, G, dv, scale, block, window, lambda, out_eps, out_scale)
+    if (dt == DT_F16) { if (maps == 1) GO(f16, 1); else GO(f16, 2); }
+    else { if (maps == 1) GO(bf16, 1); else GO(bf16, 2); }
+#undef GO
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}

@@ -90,13 +90,13 @@ extern "C" int li_activation(const float* in, void* out, int dt, int64_t n, int 
 }
 
 // ---------------------------------------------------------------------------
-// The cache of an attention whose keys are several maps wide.  A page holds PAGE tokens:
-//   keys   [kv head][token][KW]      KW = maps * d, the maps of a token side by side
-//   values [kv head][token][dv]      (the value part of a page is sized for dv rounded up to 32)
+// The cache of an attention whose keys are several maps wide.  A key of a token and KV head is its maps side by
+// side, each padded with zeros to DP = d rounded up to 16: KW = maps * DP.  Inside a page keys and values lie in
+// the order of the matrix instruction's operands (common.h, k_offset / v_offset with head size KW for the keys).
 // qk_norm_store: per token, from the float32 rows of the q/k/v product (columns q | k | v from `col0` on):
 // every map of every q and k head is divided by its root mean square over d and multiplied by a weight of size
-// d (null: none; eps < 0: no norm at all); q goes to `q_out` float32 [T, H, KW], k and v into the page of the
-// token's position.
+// d (null: none; eps < 0: no norm at all); q goes to `q_out` [T, H, KW] in the cache's type (padded likewise), k
+// and v into the page of the token's position.
 // ---------------------------------------------------------------------------
 struct MapPages {
     void* k;
@@ -109,11 +109,11 @@ struct MapPages {
 template <class T>
 __global__ void qk_norm_store_kernel(const float* __restrict__ qkv, int stride, int col0, const float* __restrict__ qw,
                                      const float* __restrict__ kw, float eps, const int* __restrict__ pos,
-                                     const int* __restrict__ tok_slot, float* __restrict__ q_out, MapPages pg, int H,
+                                     const int* __restrict__ tok_slot, T* __restrict__ q_out, MapPages pg, int H,
                                      int G, int maps, int d, int dv) {
     const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
     const float* row = qkv + (int64_t)t * stride + col0;
-    const int KW = maps * d, p = pos[t];
+    const int DP = round_up(d, 16), KW = maps * DP, p = pos[t];
     const int page = pg.page_table[(int64_t)tok_slot[t] * pg.max_pages + p / PAGE], off = p % PAGE;
     T* kp = (T*)pg.k + (int64_t)page * pg.page_stride;
     T* vp = (T*)pg.v + (int64_t)page * pg.page_stride;
@@ -125,37 +125,38 @@ __global__ void qk_norm_store_kernel(const float* __restrict__ qkv, int stride, 
         for (int i = lane; i < d; i += 64) ss += src[i] * src[i];
         const float r = eps >= 0.f ? 1.f / sqrtf(wave_sum(ss) / (float)d + eps) : 1.f;
         const float* w = is_q ? qw : kw;
-        for (int i = lane; i < d; i += 64) {
-            const float v = src[i] * r * (w ? w[i] : 1.f);
-            if (is_q) q_out[(int64_t)t * H * KW + (int64_t)u * d + i] = v;
+        for (int i = lane; i < DP; i += 64) {
+            const float v = i < d ? src[i] * r * (w ? w[i] : 1.f) : 0.f;
+            if (is_q) q_out[(int64_t)t * H * KW + (int64_t)u * DP + i] = from_f32<T>(v);
             else {
                 const int ku = u - H * maps, g = ku / maps, m = ku - g * maps;
-                kp[((int64_t)g * PAGE + off) * KW + m * d + i] = from_f32<T>(v);
+                kp[g * k_head_elems(KW) + k_offset(off, m * DP + i, KW)] = from_f32<T>(v);
             }
         }
     }
-    const float* vsrc = row + (int64_t)(H + G) * KW;
+    const float* vsrc = row + (int64_t)(H + G) * maps * d;
     for (int i = threadIdx.x; i < G * dv; i += blockDim.x) {
         const int g = i / dv, j = i - g * dv;
-        vp[((int64_t)g * PAGE + off) * dv + j] = from_f32<T>(vsrc[i]);
+        vp[g * v_head_elems(dv) + v_offset(off, j, dv)] = from_f32<T>(vsrc[i]);
     }
 }
 
 extern "C" int li_qk_norm_store(const float* qkv, int stride, int col0, const float* qw, const float* kw, float eps,
-                                const int* pos, const int* tok_slot, float* q_out, void* k_pages, void* v_pages,
+                                const int* pos, const int* tok_slot, void* q_out, void* k_pages, void* v_pages,
                                 int64_t page_stride, const int* page_table, int max_pages, int dt, int n, int H, int G,
                                 int maps, int d, int dv, hipStream_t stream) {
     if (n <= 0) return LI_OK;
     if (H <= 0 || G <= 0 || maps <= 0 || d <= 0 || dv <= 0) return LI_BAD_ARG;
     MapPages pg{k_pages, v_pages, page_stride, page_table, max_pages};
-    DISPATCH_T(dt, (qk_norm_store_kernel<T><<<n, 256, 0, stream>>>(qkv, stride, col0, qw, kw, eps, pos, tok_slot, q_out,
+    DISPATCH_T(dt, (qk_norm_store_kernel<T><<<n, 256, 0, stream>>>(qkv, stride, col0, qw, kw, eps, pos, tok_slot, (T*)q_out,
                                                                   pg, H, G, maps, d, dv)));
     LI_CHECK_LAUNCH();
     return LI_OK;
 }
 
 // ---------------------------------------------------------------------------
-// Differential attention over blocks of positions, one workgroup per (token, query head).
+// Differential attention over blocks of positions, one workgroup per (token, query head): the kernel of the
+// float32 path (the 16-bit path runs on the matrix cores, diff_attention.hip).
 // A token at position p sees the keys lo .. p with lo = p - p % block (block 0: lo = 0; window w > 0: lo is at
 // least p - w + 1).  Each of `maps` (1 or 2) maps is a softmax of its own over scores q_m . k_m * scale; with a_m
 // the maps' weighted sums of the SAME values,  o = a_1 - lambda a_2  (one map: o = a_1).  out_eps >= 0: o is
@@ -168,11 +169,11 @@ extern "C" int li_qk_norm_store(const float* qkv, int stride, int col0, const fl
 
 template <class T, int MAPS>
 __global__ __launch_bounds__(64 * DA_WAVES) void diff_attn_kernel(
-    const float* __restrict__ q, T* __restrict__ out, MapPages pg, const int* __restrict__ pos,
+    const T* __restrict__ q, T* __restrict__ out, MapPages pg, const int* __restrict__ pos,
     const int* __restrict__ tok_slot, int H, int G, int d, int dv, float scale, int block, int window, float lambda,
     float out_eps, float out_scale) {
     extern __shared__ float lds[];
-    const int KW = MAPS * d;
+    const int DP = round_up(d, 16), KW = MAPS * DP;
     float* sq = lds;                                   // [KW]
     float* sm = sq + KW;                               // [DA_WAVES][MAPS] maxima
     float* sl = sm + DA_WAVES * MAPS;                  // [DA_WAVES][MAPS] sums
@@ -182,7 +183,7 @@ __global__ __launch_bounds__(64 * DA_WAVES) void diff_attn_kernel(
     const int g = h / (H / G), p = pos[t];
     int lo = block > 0 ? p - p % block : 0;
     if (window > 0) lo = max(lo, p - window + 1);
-    for (int i = threadIdx.x; i < KW; i += blockDim.x) sq[i] = q[((int64_t)t * H + h) * KW + i];
+    for (int i = threadIdx.x; i < KW; i += blockDim.x) sq[i] = to_f32(q[((int64_t)t * H + h) * KW + i]);
     __syncthreads();
     const int* table = pg.page_table + (int64_t)tok_slot[t] * pg.max_pages;
     float m[MAPS], l[MAPS], o[MAPS][DA_MAXV];
@@ -196,20 +197,20 @@ __global__ __launch_bounds__(64 * DA_WAVES) void diff_attn_kernel(
     for (int tile = wave; tile < n_tiles; tile += DA_WAVES) {
         const int j = lo + tile * 64 + lane;           // this lane's key
         float s[MAPS];
-        const T* krow = nullptr;
-        if (j <= p) krow = (const T*)pg.k + (int64_t)table[j / PAGE] * pg.page_stride + ((int64_t)g * PAGE + j % PAGE) * KW;
+        const T* kh = nullptr;
+        if (j <= p) kh = (const T*)pg.k + (int64_t)table[j / PAGE] * pg.page_stride + g * k_head_elems(KW);
 #pragma unroll
         for (int a = 0; a < MAPS; ++a) {
             float acc = 0.f;
-            if (krow) for (int i = 0; i < d; ++i) acc += sq[a * d + i] * to_f32(krow[a * d + i]);
-            s[a] = krow ? acc * scale : -INFINITY;
+            if (kh) for (int i = 0; i < d; ++i) acc += sq[a * DP + i] * to_f32(kh[k_offset(j % PAGE, a * DP + i, KW)]);
+            s[a] = kh ? acc * scale : -INFINITY;
         }
         float pw[MAPS];
 #pragma unroll
         for (int a = 0; a < MAPS; ++a) {
             const float mt = fmaxf(m[a], wave_max(s[a]));          // lane 0's key is always visible: finite
             const float f = expf(m[a] - mt);                       // 0 the first time (m = -inf)
-            pw[a] = krow ? expf(s[a] - mt) : 0.f;
+            pw[a] = kh ? expf(s[a] - mt) : 0.f;
             l[a] = l[a] * f + wave_sum(pw[a]);
             m[a] = mt;
 #pragma unroll
@@ -218,7 +219,7 @@ __global__ __launch_bounds__(64 * DA_WAVES) void diff_attn_kernel(
         const int n_keys = min(64, p - (lo + tile * 64) + 1);
         for (int kk = 0; kk < n_keys; ++kk) {
             const int jj = lo + tile * 64 + kk;
-            const T* vrow = (const T*)pg.v + (int64_t)table[jj / PAGE] * pg.page_stride + ((int64_t)g * PAGE + jj % PAGE) * dv;
+            const T* vh = (const T*)pg.v + (int64_t)table[jj / PAGE] * pg.page_stride + g * v_head_elems(dv);
             float w[MAPS];
 #pragma unroll
             for (int a = 0; a < MAPS; ++a) w[a] = __shfl(pw[a], kk, WAVE);
@@ -226,7 +227,7 @@ __global__ __launch_bounds__(64 * DA_WAVES) void diff_attn_kernel(
             for (int c = 0; c < DA_MAXV; ++c) {
                 const int i = lane + 64 * c;
                 if (i < dv) {
-                    const float v = to_f32(vrow[i]);
+                    const float v = to_f32(vh[v_offset(jj % PAGE, i, dv)]);
 #pragma unroll
                     for (int a = 0; a < MAPS; ++a) o[a][c] += w[a] * v;
                 }
@@ -283,7 +284,7 @@ __global__ __launch_bounds__(64 * DA_WAVES) void diff_attn_kernel(
     }
 }
 
-extern "C" int li_diff_attn(const float* q, void* out, int dt, void* k_pages, void* v_pages, int64_t page_stride,
+extern "C" int li_diff_attn(const void* q, void* out, int dt, void* k_pages, void* v_pages, int64_t page_stride,
                             const int* page_table, int max_pages, const int* pos, const int* tok_slot, int n, int H, int G,
                             int maps, int d, int dv, float scale, int block, int window, float lambda, float out_eps,
                             float out_scale, hipStream_t stream) {
@@ -292,10 +293,10 @@ extern "C" int li_diff_attn(const float* q, void* out, int dt, void* k_pages, vo
     if (maps < 1 || maps > 2 || dv > 64 * DA_MAXV) return LI_UNSUPPORTED;
     MapPages pg{k_pages, v_pages, page_stride, page_table, max_pages};
     dim3 grid(n, H), blk(64 * DA_WAVES);
-    const size_t lds = (size_t)(maps * d + 2 * DA_WAVES * maps + DA_WAVES * maps * dv) * sizeof(float);
+    const size_t lds = (size_t)(maps * round_up(d, 16) + 2 * DA_WAVES * maps + DA_WAVES * maps * dv) * sizeof(float);
     if (lds > 60000) return LI_UNSUPPORTED;
-#define GO(M) diff_attn_kernel<T, M><<<grid, blk, lds, stream>>>(q, (T*)out, pg, pos, tok_slot, H, G, d, dv, scale, block, \
-                                                                 window, lambda, out_eps, out_scale)
+#define GO(M) diff_attn_kernel<T, M><<<grid, blk, lds, stream>>>((const T*)q, (T*)out, pg, pos, tok_slot, H, G, d, dv, scale, \
+                                                                 block, window, lambda, out_eps, out_scale)
     DISPATCH_T(dt, { if (maps == 1) GO(1); else GO(2); });
 #undef GO
     LI_CHECK_LAUNCH();
@@ -320,7 +321,7 @@ __global__ void conv_silu_kernel(const float* __restrict__ in, int stride, int c
     int inside = 0;
     while (inside < taps - 1 && t - inside - 1 >= 0 && tok_slot[t - inside - 1] == slot) ++inside;
     const float* h = hist + (int64_t)slot * (taps - 1) * channels;
-    for (int c = threadIdx.x; c < channels; c += blockDim.x) {
+    for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < channels; c += gridDim.y * blockDim.x) {
         float acc = b ? b[c] : 0.f;
         for (int back = 0; back < taps; ++back) {                  // back = taps - 1 - j
             float u = 0.f;
@@ -354,7 +355,8 @@ extern "C" int li_conv_silu(const float* in, int stride, int col0, const float* 
                             hipStream_t stream) {
     if (n_tokens <= 0) return LI_OK;
     if (channels <= 0 || taps < 1 || taps > CONV_MAX_TAPS) return LI_BAD_ARG;
-    conv_silu_kernel<<<n_tokens, 256, 0, stream>>>(in, stride, col0, w, b, hist, pos, tok_slot, out, channels, taps);
+    dim3 cgrid(n_tokens, (channels + 255) / 256);
+    conv_silu_kernel<<<cgrid, 256, 0, stream>>>(in, stride, col0, w, b, hist, pos, tok_slot, out, channels, taps);
     if (taps > 1) {
         dim3 grid(n_seqs, (channels + 255) / 256);
         conv_history_kernel<<<grid, 256, 0, stream>>>(in, stride, col0, hist, seq_slot, seq_qstart, seq_qlen, channels, taps);
@@ -370,54 +372,121 @@ extern "C" int li_conv_silu(const float* in, int stride, int col0, const float* 
 //   S <- a S + dt B_t x_t^T   (S is N x dv, float32, kept for every sequence in `state` [slots, P, N, dv])
 //   y_t = S^T C_t + D[h] x_t
 // One wave per (sequence, head, 64 columns of dv): a lane keeps its column of S in registers for all the tokens
-// that the sequence brings; B_t and C_t reach the lanes through LDS, fetched a token ahead.
+// that the sequence brings; B_t and C_t lie across the lanes and reach every lane by lane reads.
 // ---------------------------------------------------------------------------
-template <int NMAX>
+// A prompt may also be walked in segments (ScanPlan): pass 1 runs every segment from a zero state and leaves its own
+// contribution and the product of its decays; ssm_combine_kernel walks a sequence's segments in order, S <- a_seg S +
+// D_seg, leaving the state before every segment where its contribution was; pass 3 runs every segment again from
+// that state and writes y.  Twice the arithmetic, and as many waves as there are segments instead of sequences.
+struct ScanPlan {
+    int pass;                   // 0: a sequence's tokens in order; 1 and 3: see above
+    const int* seg_seq;         // [segments] the sequence of a segment
+    const int* seg_t0;          // [segments] its first token among the sequence's tokens of this step
+    const int* seg_n;           // [segments] its tokens
+    float* seg_state;           // [segments, P, N, dv]
+    float* seg_decay;           // [segments, P]
+};
+
+template <int NMAX, int PASS>
 __global__ __launch_bounds__(64) void ssm_scan_kernel(
     const float* __restrict__ xbc, int xbc_stride, const float* __restrict__ proj, int proj_stride, int dt_col,
     const float* __restrict__ dt_bias, const float* __restrict__ A_log, const float* __restrict__ D,
     float* __restrict__ state, const int* __restrict__ seq_slot, const int* __restrict__ seq_qstart,
-    const int* __restrict__ seq_qlen, float* __restrict__ y, int P, int G, int N, int dv) {
-    __shared__ float sb[2][2 * NMAX];                       // [stage][B | C]
-    const int seq = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, col = blockIdx.z * 64 + lane;
+    const int* __restrict__ seq_qlen, float* __restrict__ y, int P, int G, int N, int dv, ScanPlan plan) {
+    const int h = blockIdx.y, lane = threadIdx.x, col = blockIdx.z * 64 + lane;
     const int g = h / (P / G), inner = P * dv;
-    const int q0 = seq_qstart ? seq_qstart[seq] : seq, n = seq_qlen ? seq_qlen[seq] : 1;
+    int q0, n;
+    float* S;
+    if (PASS == 0) {
+        const int seq = blockIdx.x;
+        q0 = seq_qstart ? seq_qstart[seq] : seq;
+        n = seq_qlen ? seq_qlen[seq] : 1;
+        S = state + (((int64_t)seq_slot[seq] * P + h) * N) * dv + col;
+    } else {
+        const int seg = blockIdx.x;
+        q0 = seq_qstart[plan.seg_seq[seg]] + plan.seg_t0[seg];
+        n = plan.seg_n[seg];
+        S = plan.seg_state + (((int64_t)seg * P + h) * N) * dv + col;
+    }
     const bool live = col < dv;
-    float* S = state + (((int64_t)seq_slot[seq] * P + h) * N) * dv + col;
     float s[NMAX];
 #pragma unroll
-    for (int i = 0; i < NMAX; ++i) s[i] = (live && i < N) ? S[(int64_t)i * dv] : 0.f;
+    for (int i = 0; i < NMAX; ++i) s[i] = (live && i < N && PASS != 1) ? S[(int64_t)i * dv] : 0.f;
     const float negA = -expf(A_log[h]), bias = dt_bias[h], dh = D ? D[h] : 0.f;
     const int b_off = inner + g * N, c_off = inner + G * N + g * N;
-    auto fetch = [&](int t, int stage) {
-        const float* row = xbc + (int64_t)(q0 + t) * xbc_stride;
-        for (int i = lane; i < N; i += 64) { sb[stage][i] = row[b_off + i]; sb[stage][NMAX + i] = row[c_off + i]; }
+    float log_decay = 0.f;
+    // B_t and C_t are the same for all lanes: lane j fetches elements j, j + 64, ... (a token ahead, so that the wait for
+    // memory lies under the token at work), and element i reaches all lanes by a lane read, which costs no memory
+    // or LDS bandwidth.  Elements from N on are zero and leave the state's zeros as they are.
+    constexpr int NV = (NMAX + 63) / 64;
+    float bv[NV], cv[NV], x = 0.f, dt = 0.f;
+    auto fetch = [&](int t) {
+        const float* __restrict__ row = xbc + (int64_t)(q0 + t) * xbc_stride;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int i = v * 64 + lane;
+            bv[v] = i < N ? row[b_off + i] : 0.f;
+            cv[v] = i < N ? row[c_off + i] : 0.f;
+        }
+        x = live ? row[h * dv + col] : 0.f;
+        dt = proj[(int64_t)(q0 + t) * proj_stride + dt_col + h];
     };
-    if (n > 0) fetch(0, 0);
-    __syncthreads();
+    if (n > 0) fetch(0);
     for (int t = 0; t < n; ++t) {
-        const int stage = t & 1;
-        if (t + 1 < n) fetch(t + 1, stage ^ 1);
-        const float dt = softplusf_(proj[(int64_t)(q0 + t) * proj_stride + dt_col + h] + bias);
-        const float a = expf(negA * dt);
-        const float x = live ? xbc[(int64_t)(q0 + t) * xbc_stride + h * dv + col] : 0.f;
-        const float dx = dt * x;
+        float bt[NV], ct[NV];
+#pragma unroll
+        for (int v = 0; v < NV; ++v) { bt[v] = bv[v]; ct[v] = cv[v]; }
+        const float xt = x, dtt = softplusf_(dt + bias);
+        if (t + 1 < n) fetch(t + 1);
+        const float lda = negA * dtt, a = expf(lda);
+        log_decay += lda;
+        const float dx = dtt * xt;
         float acc = 0.f;
 #pragma unroll
         for (int i = 0; i < NMAX; ++i) {
-            if (i < N) {
-                s[i] = a * s[i] + sb[stage][i] * dx;
-                acc += s[i] * sb[stage][NMAX + i];
+            const float b = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(bt[i >> 6]), i & 63));
+            s[i] = a * s[i] + b * dx;
+            if (PASS != 1) {
+                const float c = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(ct[i >> 6]), i & 63));
+                acc += s[i] * c;
             }
         }
-        if (live) y[(int64_t)(q0 + t) * inner + h * dv + col] = acc + dh * x;
-        __syncthreads();
+        if (live && PASS != 1) y[(int64_t)(q0 + t) * inner + h * dv + col] = acc + dh * xt;
     }
-    if (live) {
+    if (live && PASS != 3) {
 #pragma unroll
         for (int i = 0; i < NMAX; ++i) if (i < N) S[(int64_t)i * dv] = s[i];
     }
+    if (PASS == 1 && lane == 0 && blockIdx.z == 0) plan.seg_decay[(int64_t)blockIdx.x * P + h] = expf(log_decay);
 }
+
+// One thread per element of a head's state: walks the sequence's segments in order.
+__global__ void ssm_combine_kernel(float* __restrict__ state, const int* __restrict__ seq_slot,
+                                   const int* __restrict__ seq_seg0, const int* __restrict__ seq_nseg,
+                                   float* __restrict__ seg_state, const float* __restrict__ seg_decay, int P, int64_t per_head) {
+    const int seq = blockIdx.x, h = blockIdx.y;
+    const int c0 = seq_seg0[seq], nc = seq_nseg[seq];
+    for (int64_t e = (int64_t)blockIdx.z * blockDim.x + threadIdx.x; e < per_head; e += (int64_t)gridDim.z * blockDim.x) {
+        float* S = state + ((int64_t)seq_slot[seq] * P + h) * per_head + e;
+        float s = *S;
+        for (int c = c0; c < c0 + nc; ++c) {
+            float* L = seg_state + ((int64_t)c * P + h) * per_head + e;
+            const float own = *L;
+            *L = s;
+            s = seg_decay[(int64_t)c * P + h] * s + own;
+        }
+        *S = s;
+    }
+}
+
+#define SSM_GO(NM, GRID, PLAN) ssm_scan_kernel<NM, SSM_PASS><<<GRID, 64, 0, stream>>>(xbc, xbc_stride, proj, proj_stride, dt_col, \
+        dt_bias, A_log, D, state, seq_slot, seq_qstart, seq_qlen, y, P, G, N, dv, PLAN)
+#define SSM_LAUNCH(GRID, PLAN)                                                                  \
+    do {                                                                                        \
+        if (N <= 16) SSM_GO(16, GRID, PLAN); else if (N <= 32) SSM_GO(32, GRID, PLAN);          \
+        else if (N <= 64) SSM_GO(64, GRID, PLAN); else if (N <= 128) SSM_GO(128, GRID, PLAN);   \
+        else SSM_GO(256, GRID, PLAN);                                                           \
+    } while (0)
 
 extern "C" int li_ssm_scan(const float* xbc, int xbc_stride, const float* proj, int proj_stride, int dt_col,
                            const float* dt_bias, const float* A_log, const float* D, float* state, const int* seq_slot,
@@ -427,10 +496,37 @@ extern "C" int li_ssm_scan(const float* xbc, int xbc_stride, const float* proj, 
     if (P <= 0 || G <= 0 || P % G || N <= 0 || dv <= 0) return LI_BAD_ARG;
     if (N > 256) return LI_UNSUPPORTED;
     dim3 grid(n_seqs, P, (dv + 63) / 64);
-#define GO(NM) ssm_scan_kernel<NM><<<grid, 64, 0, stream>>>(xbc, xbc_stride, proj, proj_stride, dt_col, dt_bias, A_log, D, \
-                                                            state, seq_slot, seq_qstart, seq_qlen, y, P, G, N, dv)
-    if (N <= 16) GO(16); else if (N <= 32) GO(32); else if (N <= 64) GO(64); else if (N <= 128) GO(128); else GO(256);
-#undef GO
+    ScanPlan plan{0, nullptr, nullptr, nullptr, nullptr, nullptr};
+#define SSM_PASS 0
+    SSM_LAUNCH(grid, plan);
+#undef SSM_PASS
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// The same recurrence with every sequence's tokens cut into segments that run side by side (see ScanPlan).
+// seg_state [segments, P, N, dv] and seg_decay [segments, P] are scratch memory of the caller.
+extern "C" int li_ssm_scan_segments(const float* xbc, int xbc_stride, const float* proj, int proj_stride, int dt_col,
+                                    const float* dt_bias, const float* A_log, const float* D, float* state,
+                                    const int* seq_slot, const int* seq_qstart, const int* seq_qlen, float* y, int n_seqs,
+                                    int P, int G, int N, int dv, const int* seg_seq, const int* seg_t0, const int* seg_n,
+                                    const int* seq_seg0, const int* seq_nseg, int n_segs, float* seg_state, float* seg_decay,
+                                    hipStream_t stream) {
+    if (n_seqs <= 0 || n_segs <= 0) return LI_OK;
+    if (P <= 0 || G <= 0 || P % G || N <= 0 || dv <= 0 || !seq_qstart || !seq_qlen) return LI_BAD_ARG;
+    if (N > 256) return LI_UNSUPPORTED;
+    dim3 grid(n_segs, P, (dv + 63) / 64);
+    ScanPlan plan{1, seg_seq, seg_t0, seg_n, seg_state, seg_decay};
+#define SSM_PASS 1
+    SSM_LAUNCH(grid, plan);
+#undef SSM_PASS
+    const int64_t per_head = (int64_t)N * dv;
+    dim3 cgrid(n_seqs, P, (unsigned)((per_head + 255) / 256));
+    ssm_combine_kernel<<<cgrid, 256, 0, stream>>>(state, seq_slot, seq_seg0, seq_nseg, seg_state, seg_decay, P, per_head);
+    plan.pass = 3;
+#define SSM_PASS 3
+    SSM_LAUNCH(grid, plan);
+#undef SSM_PASS
     LI_CHECK_LAUNCH();
     return LI_OK;
 }
@@ -459,7 +555,43 @@ extern "C" int li_gated_group_norm(const float* y, const float* zrows, int z_str
     if (n_rows <= 0) return LI_OK;
     if (n <= 0 || groups <= 0 || n % groups) return LI_BAD_ARG;
     dim3 grid(n_rows, groups);
-    DISPATCH_T(dt, (gated_group_norm_kernel<T><<<grid, 256, 0, stream>>>(y, zrows, z_stride, z_col, w, (T*)out, n, groups, eps)));
+    const int threads = n / groups >= 4096 ? 1024 : (n / groups >= 1024 ? 512 : 256);
+    DISPATCH_T(dt, (gated_group_norm_kernel<T><<<grid, threads, 0, stream>>>(y, zrows, z_stride, z_col, w, (T*)out, n, groups, eps)));
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// out[t][j] = w[j] . h[t] in float32 for a few rows of a float32 matrix w [n, width] (a router's): one
+// wave per (token, output), the lanes stride the width; every sum has one fixed order whatever the batch.
+// ---------------------------------------------------------------------------
+template <class T>
+__global__ __launch_bounds__(64) void small_logits_kernel(const T* __restrict__ h, const float* __restrict__ w,
+                                                          float* __restrict__ out, int width, int n) {
+    const int t = blockIdx.x, j = blockIdx.y, lane = threadIdx.x;
+    const T* row = h + (int64_t)t * width;
+    const float* wj = w + (int64_t)j * width;
+    float part[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) part[u] = 0.f;
+    for (int i0 = 0; i0 < width; i0 += 512) {              // eight independent loads of each operand at a time
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = i0 + u * 64 + lane;
+            if (i < width) part[u] += wj[i] * to_f32(row[i]);
+        }
+    }
+    float acc = ((part[0] + part[1]) + (part[2] + part[3])) + ((part[4] + part[5]) + (part[6] + part[7]));
+    acc = wave_sum(acc);
+    if (lane == 0) out[(int64_t)t * n + j] = acc;
+}
+
+extern "C" int li_small_logits(const void* h, int dt, const float* w, float* out, int n_rows, int width, int n,
+                               hipStream_t stream) {
+    if (n_rows <= 0 || n <= 0) return LI_OK;
+    if (width <= 0 || n > 65535) return LI_BAD_ARG;
+    dim3 grid(n_rows, n);
+    DISPATCH_T(dt, (small_logits_kernel<T><<<grid, 64, 0, stream>>>((const T*)h, w, out, width, n)));
     LI_CHECK_LAUNCH();
     return LI_OK;
 }
@@ -547,7 +679,7 @@ template <class T>
 __global__ void scale_blocks_kernel(T* __restrict__ t, const float* __restrict__ weights, int n_blocks, int ff, int tail) {
     const int64_t row = blockIdx.x;
     const int cols = n_blocks * ff + tail, wcols = n_blocks + (tail ? 1 : 0);
-    for (int i = threadIdx.x; i < cols; i += blockDim.x) {
+    for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < cols; i += gridDim.y * blockDim.x) {
         const int e = i < n_blocks * ff ? i / ff : n_blocks;
         const float w = weights[row * wcols + e];
         t[row * cols + i] = from_f32<T>(w == 0.f ? 0.f : to_f32(t[row * cols + i]) * w);
@@ -558,7 +690,79 @@ extern "C" int li_scale_blocks(void* t, int dt, const float* weights, int n, int
                                hipStream_t stream) {
     if (n <= 0) return LI_OK;
     if (n_blocks < 0 || ff < 0 || tail < 0) return LI_BAD_ARG;
-    DISPATCH_T(dt, (scale_blocks_kernel<T><<<n, 256, 0, stream>>>((T*)t, weights, n_blocks, ff, tail)));
+    const int cols = n_blocks * ff + tail;
+    dim3 grid(n, n >= 1024 ? 1 : (cols + 1023) / 1024);        // few rows: the columns over the grid as well
+    DISPATCH_T(dt, (scale_blocks_kernel<T><<<grid, 256, 0, stream>>>((T*)t, weights, n_blocks, ff, tail)));
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Tokens sorted by expert, for prompts long enough that every expert gets a product of its own.
+// moe_bucket_kernel: workgroup e lists, in ascending order, the tokens whose weight for expert e is not zero
+// (idx [E, T]) and counts them (counts [E]).  gather_rows: out[r] = h[idx[r]].  scatter_add_rows:
+// residual[idx[r]] += weights[idx[r]][col] * y[r]  (idx null: row r itself).
+// ---------------------------------------------------------------------------
+__global__ void moe_bucket_kernel(const float* __restrict__ weights, int wcols, int n_tokens, int* __restrict__ idx,
+                                  int* __restrict__ counts) {
+    __shared__ int part[256];
+    const int e = blockIdx.x, tid = threadIdx.x;
+    const int per = (n_tokens + 255) / 256, lo = min(n_tokens, tid * per), hi = min(n_tokens, lo + per);
+    int mine = 0;
+    for (int t = lo; t < hi; ++t) mine += weights[(int64_t)t * wcols + e] != 0.f;
+    part[tid] = mine;
+    __syncthreads();
+    if (tid == 0) {
+        int run = 0;
+        for (int i = 0; i < 256; ++i) { const int c = part[i]; part[i] = run; run += c; }
+        counts[e] = run;
+    }
+    __syncthreads();
+    int at = part[tid];
+    for (int t = lo; t < hi; ++t)
+        if (weights[(int64_t)t * wcols + e] != 0.f) idx[(int64_t)e * n_tokens + at++] = t;
+}
+
+extern "C" int li_moe_buckets(const float* weights, int wcols, int n_tokens, int n_experts, int* idx, int* counts,
+                              hipStream_t stream) {
+    if (n_tokens <= 0 || n_experts <= 0) return LI_OK;
+    if (wcols < n_experts) return LI_BAD_ARG;
+    moe_bucket_kernel<<<n_experts, 256, 0, stream>>>(weights, wcols, n_tokens, idx, counts);
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+template <class T>
+__global__ void gather_rows_kernel(const T* __restrict__ h, const int* __restrict__ idx, T* __restrict__ out, int width) {
+    const int64_t r = blockIdx.x, src = idx[r];
+    for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < width; i += gridDim.y * blockDim.x)
+        out[r * width + i] = h[src * width + i];
+}
+
+extern "C" int li_gather_rows(const void* h, int dt, const int* idx, void* out, int n, int width, hipStream_t stream) {
+    if (n <= 0) return LI_OK;
+    if (width <= 0) return LI_BAD_ARG;
+    dim3 grid(n, n >= 1024 ? 1 : (width + 1023) / 1024);
+    DISPATCH_T(dt, (gather_rows_kernel<T><<<grid, 256, 0, stream>>>((const T*)h, idx, (T*)out, width)));
+    LI_CHECK_LAUNCH();
+    return LI_OK;
+}
+
+__global__ void scatter_add_rows_kernel(float* __restrict__ residual, const float* __restrict__ y,
+                                        const int* __restrict__ idx, const float* __restrict__ weights, int wcols, int col,
+                                        int width) {
+    const int64_t r = blockIdx.x, dst = idx ? idx[r] : r;
+    const float w = weights[dst * wcols + col];
+    for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < width; i += gridDim.y * blockDim.x)
+        residual[dst * width + i] += w * y[r * width + i];
+}
+
+extern "C" int li_scatter_add_rows(float* residual, const float* y, const int* idx, const float* weights, int wcols,
+                                   int col, int n, int width, hipStream_t stream) {
+    if (n <= 0) return LI_OK;
+    if (width <= 0 || col < 0 || col >= wcols) return LI_BAD_ARG;
+    dim3 grid(n, n >= 1024 ? 1 : (width + 1023) / 1024);
+    scatter_add_rows_kernel<<<grid, 256, 0, stream>>>(residual, y, idx, weights, wcols, col, width);
     LI_CHECK_LAUNCH();
     return LI_OK;
 }

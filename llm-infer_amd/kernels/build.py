@@ -200,6 +200,23 @@ def hybrid_library(force=False):
     return _load("libli_hybrid.so", HYBRID_SOURCES, (), force)
 
 
+DIFF_ATTN_SOURCE = "diff_attention.hip"
+
+
+def _diff_attention_args(map_dim: int, value_dim: int):
+    if map_dim % 16 != 0 or not 16 <= map_dim <= 256 or value_dim % 32 != 0 or not 32 <= value_dim <= 256:
+        raise BuildError(f"head sizes {map_dim} / {value_dim}: the differential attention kernel takes a map size that is "
+                         "a multiple of 16 and a value size that is a multiple of 32, both up to 256")
+    return (f"libli_diffattn_k{map_dim}_v{value_dim}.so", (DIFF_ATTN_SOURCE,),
+            (f"-DMAP_DIM={map_dim}", f"-DVALUE_DIM={value_dim}"))
+
+
+def diff_attention_library(map_dim: int, value_dim: int, force=False):
+    """The matrix-core kernel of differential attention for one pair of sizes (a map's keys, values), compiled at
+    the first call that needs the pair."""
+    return _load(*_diff_attention_args(map_dim, value_dim), force)
+
+
 SIGMOID_ATTN_SOURCE = "sigmoid_attention.hip"
 
 
@@ -217,7 +234,8 @@ def sigmoid_attention_library(key_dim: int, value_dim: int, force=False):
     return _load(*_sigmoid_attention_args(key_dim, value_dim), force)
 
 
-def build_all(head_dims=(16, 32, 48, 64, 128), force=True, sigmoid_head_dims=((48, 32), (128, 128))) -> None:
+def build_all(head_dims=(16, 32, 48, 64, 128), force=True, sigmoid_head_dims=((48, 32), (128, 128)),
+              diff_head_dims=((32, 64), (64, 128))) -> None:
     """Compile the core library, the mixers' library, the attention library for each head size given and the
     sigmoid attention library for each pair of head sizes given."""
     core_library(force=force)
@@ -225,6 +243,7 @@ def build_all(head_dims=(16, 32, 48, 64, 128), force=True, sigmoid_head_dims=((4
     hybrid_library(force=force)
     with ThreadPoolExecutor(max_workers=4) as pool:
         list(pool.map(lambda p: _build_library(*_sigmoid_attention_args(*p), force), sigmoid_head_dims))
+        list(pool.map(lambda p: _build_library(*_diff_attention_args(*p), force), diff_head_dims))
     with ThreadPoolExecutor(max_workers=4) as pool:
         list(pool.map(lambda hd: _build_library(f"libli_attn_hd{hd}.so", (ATTN_SOURCE,),
                                                 (f"-DHEAD_DIM={hd}",), force), head_dims))

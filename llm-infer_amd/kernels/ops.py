@@ -1162,31 +1162,37 @@ def activation(z, kind: str, out_dtype) -> torch.Tensor:
     return out
 
 
+def padded_map_dim(d: int) -> int:
+    """The width of one map's keys in the pages and in q: the next multiple of 16 (zeros behind the d dimensions)."""
+    return (d + 15) // 16 * 16
+
+
 def _map_pages_check(kv, n_kv_heads, key_width, v_dim):
     k_pages, v_pages, page_stride, page_table = kv
     _dev(k_pages, v_pages, page_table)
     _need(k_pages.dtype == v_pages.dtype and k_pages.dtype in DT, "cache: one float type for keys and values")
     _need(page_table.dtype == torch.int32 and page_table.dim() == 2, "page_table: int32 [slots, pages]")
-    _need(page_stride >= n_kv_heads * PAGE * (key_width + v_dim), "a page is too small for these keys and values")
+    _need(page_stride >= n_kv_heads * PAGE * (key_width + (v_dim + 31) // 32 * 32), "a page is too small for these keys and values")
     return k_pages, v_pages, page_stride, page_table
 
 
 def qk_norm_store(qkv, col0, q_weight, k_weight, eps, pos, tok_slot, kv, n_heads, n_kv_heads, maps, d, dv) -> torch.Tensor:
     """From the float32 rows of a q/k/v product (columns from ``col0``: q [H, maps, d] | k [G, maps, d] | v [G, dv]):
     each map of each q and k head divided by its root mean square over d and multiplied by a weight [d] (``eps``
-    None: no norm); returns q float32 [T, H, maps * d]; k and v go into the pages (keys [head][token][maps * d],
-    values [head][token][dv]) at each token's position."""
+    None: no norm).  Returns q [T, H, maps * DP] in the cache's type, DP = ``padded_map_dim(d)`` with zeros behind
+    a map's d dimensions; k (padded likewise) and v go into the pages in matrix-operand order (csrc/common.h, keys
+    of head size maps * DP) at each token's position."""
     _dev(qkv, q_weight, k_weight, pos, tok_slot)
     _f32_rows(qkv, "qk_norm_store rows")
     t = qkv.shape[0]
-    kw = maps * d
-    _need(col0 >= 0 and col0 + (n_heads + n_kv_heads) * kw + n_kv_heads * dv <= qkv.shape[1], "qk_norm_store: columns beyond the rows")
+    kw = maps * padded_map_dim(d)
+    _need(col0 >= 0 and col0 + (n_heads + n_kv_heads) * maps * d + n_kv_heads * dv <= qkv.shape[1], "qk_norm_store: columns beyond the rows")
     for w in (q_weight, k_weight):
         _need(w is None or (w.dtype == torch.float32 and w.shape == (d,)), "q/k norm weight: float32 [d]")
     _i32(pos, t, "positions")
     _i32(tok_slot, t, "slots")
     k_pages, v_pages, page_stride, page_table = _map_pages_check(kv, n_kv_heads, kw, dv)
-    q = torch.empty((t, n_heads, kw), dtype=torch.float32, device=qkv.device)
+    q = torch.empty((t, n_heads, kw), dtype=k_pages.dtype, device=qkv.device)
     _check(hybrid().li_qk_norm_store(_ptr(qkv), qkv.shape[1], col0, _ptr(q_weight), _ptr(k_weight),
                                      c_float(-1.0 if eps is None else eps), _ptr(pos), _ptr(tok_slot), _ptr(q), _ptr(k_pages),
                                      _ptr(v_pages), c_int64(page_stride), _ptr(page_table), page_table.shape[1],
@@ -1194,25 +1200,84 @@ def qk_norm_store(qkv, col0, q_weight, k_weight, eps, pos, tok_slot, kv, n_heads
     return q
 
 
+DIFF_TILE = 32            # tokens of one wave of the matrix-core differential attention
+_diffattn: dict = {}
+
+
+def _diffattn_lib(map_dim: int, value_dim: int):
+    lib = _diffattn.get((map_dim, value_dim))
+    if lib is None:
+        lib = build.diff_attention_library(map_dim, value_dim)
+        _need(lib.li_diffattn_map_dim() == map_dim and lib.li_diffattn_value_dim() == value_dim,
+              "differential attention library built for other head sizes")
+        _diffattn[map_dim, value_dim] = lib
+    return lib
+
+
+def diff_tiles(ctx):
+    """The tiles of the matrix-core differential attention for a step: up to DIFF_TILE consecutive tokens of one
+    sequence each, as int32 device arrays (first row, rows) and their number; made once per step and shared.
+    None for a step in which every sequence brings one token (every token is then a tile of its own)."""
+    if ctx.n_tokens == ctx.n_seqs or getattr(ctx, "host_qlens", None) is None:
+        return None
+
+    def make():
+        t0, n, at = [], [], 0
+        for q in ctx.host_qlens:
+            for lo in range(0, q, DIFF_TILE):
+                t0.append(at + lo)
+                n.append(min(DIFF_TILE, q - lo))
+            at += q
+        both = torch.tensor([t0, n], dtype=torch.int32).to(ctx.device)
+        return both[0], both[1], len(t0)
+    return ctx.shared(("diff_attention_tiles", DIFF_TILE), make)
+
+
 def diff_attention(q, kv, pos, tok_slot, n_heads, n_kv_heads, maps, d, dv, scale, block, window, lam, out_eps, out_scale,
-                   out_dtype) -> torch.Tensor:
+                   out_dtype, tiles=None) -> torch.Tensor:
     """Attention of ``maps`` softmax maps (1 or 2) over the same values: o = a_1 - lam a_2, then (``out_eps`` not
     None) o divided by its root mean square over dv, times ``out_scale``.  A token at position p sees the keys
-    from p - p % block on (``block`` 0: from 0; ``window`` w: at most the last w).  q float32 [T, H, maps * d];
-    returns [T, H * dv] in ``out_dtype``."""
+    from p - p % block on (``block`` 0: from 0; ``window`` w: at most the last w).  q [T, H, maps * DP] as
+    ``qk_norm_store`` leaves it; returns [T, H * dv] in ``out_dtype``, the cache's type.  A float32 cache runs one
+    workgroup per (token, head); a 16-bit cache runs on the matrix cores, one wave per (tile, head) with ``tiles``
+    from ``diff_tiles`` (None: every token a tile of its own)."""
     _dev(q, pos, tok_slot)
     t = q.shape[0]
-    _need(q.dtype == torch.float32 and q.shape == (t, n_heads, maps * d), "q: float32 [T, H, maps * d]")
+    dp = padded_map_dim(d)
     _need(maps in (1, 2) and dv <= 256 and n_heads % n_kv_heads == 0, "diff_attention: one or two maps, values up to 256 wide")
     _i32(pos, t, "positions")
     _i32(tok_slot, t, "slots")
-    k_pages, v_pages, page_stride, page_table = _map_pages_check(kv, n_kv_heads, maps * d, dv)
+    k_pages, v_pages, page_stride, page_table = _map_pages_check(kv, n_kv_heads, maps * dp, dv)
+    _need(q.dtype == k_pages.dtype and q.shape == (t, n_heads, maps * dp), "q: [T, H, maps * DP] in the cache's type")
     _need(out_dtype == k_pages.dtype, "diff_attention: the output has the cache's type")
     out = torch.empty((t, n_heads * dv), dtype=out_dtype, device=q.device)
-    _check(hybrid().li_diff_attn(_ptr(q), _ptr(out), DT[out_dtype], _ptr(k_pages), _ptr(v_pages), c_int64(page_stride),
-                                 _ptr(page_table), page_table.shape[1], _ptr(pos), _ptr(tok_slot), t, n_heads, n_kv_heads,
-                                 maps, d, dv, c_float(scale), int(block or 0), int(window or 0), c_float(lam),
-                                 c_float(-1.0 if out_eps is None else out_eps), c_float(out_scale), _stream()), "diff_attn")
+    tail = (c_float(scale), int(block or 0), int(window or 0), c_float(lam), c_float(-1.0 if out_eps is None else out_eps),
+            c_float(out_scale), _stream())
+    if out_dtype == torch.float32:
+        _check(hybrid().li_diff_attn(_ptr(q), _ptr(out), DT[out_dtype], _ptr(k_pages), _ptr(v_pages), c_int64(page_stride),
+                                     _ptr(page_table), page_table.shape[1], _ptr(pos), _ptr(tok_slot), t, n_heads, n_kv_heads,
+                                     maps, d, dv, *tail), "diff_attn")
+        return out
+    _need(dp <= 256, "diff_attention on the matrix cores: a map's keys up to 256 wide")
+    tile_t0, tile_n, n_tiles = tiles if tiles is not None else (None, None, t)
+    if tiles is not None:
+        _i32(tile_t0, n_tiles, "tile starts")
+        _i32(tile_n, n_tiles, "tile sizes")
+    _check(_diffattn_lib(dp, (dv + 31) // 32 * 32).li_diffattn(
+        _ptr(q), _ptr(out), DT[out_dtype], _ptr(k_pages), _ptr(v_pages), c_int64(page_stride), _ptr(page_table),
+        page_table.shape[1], _ptr(pos), _ptr(tok_slot), _ptr(tile_t0), _ptr(tile_n), n_tiles, n_heads, n_kv_heads, maps, dv,
+        *tail), "diffattn")
+    return out
+
+
+def small_logits(h, w) -> torch.Tensor:
+    """h W^T in float32 for a float32 matrix of a few rows (a router's): every sum in one fixed order."""
+    _dev(h, w)
+    _need(h.dim() == 2 and h.dtype in DT and w.dtype == torch.float32 and w.dim() == 2 and w.shape[1] == h.shape[1],
+          "small_logits: h [T, width], a float32 matrix [n, width]")
+    out = torch.empty((h.shape[0], w.shape[0]), dtype=torch.float32, device=h.device)
+    _check(hybrid().li_small_logits(_ptr(h), DT[h.dtype], _ptr(w), _ptr(out), h.shape[0], h.shape[1], w.shape[0], _stream()),
+           "small_logits")
     return out
 
 
@@ -1240,10 +1305,36 @@ def conv_silu(rows, col0, channels, weight, bias, history, ctx) -> torch.Tensor:
     return out
 
 
-def ssm_scan(xbc, proj, dt_col, dt_bias, a_log, d_skip, state, ctx, heads, groups, n_state, dv) -> torch.Tensor:
-    """The selective state-space recurrence, token by token in float32.  ``xbc`` float32 [T, heads * dv + 2 groups
-    n_state] (x | B | C), the raw step sizes in ``proj`` columns dt_col .. dt_col + heads; ``state`` float32
-    [slots, heads, n_state, dv], read and left up to date; returns y float32 [T, heads * dv]."""
+SSM_SEGMENT = 128          # tokens of a segment when a prompt's recurrence runs in segments side by side
+
+
+def ssm_segments(ctx, length: int | None = None) -> dict:
+    """The segments of a step's sequences for ``ssm_scan`` (made once per step and shared): every sequence's tokens
+    cut every ``length`` tokens; int32 device arrays seg_seq, seg_t0, seg_n, seq_seg0, seq_nseg and the count."""
+    length = length or SSM_SEGMENT
+
+    def make():
+        seg_seq, seg_t0, seg_n, seq_seg0, seq_nseg = [], [], [], [], []
+        for i, n in enumerate(ctx.host_qlens):
+            seq_seg0.append(len(seg_seq))
+            for t0 in range(0, n, length):
+                seg_seq.append(i)
+                seg_t0.append(t0)
+                seg_n.append(min(length, n - t0))
+            seq_nseg.append(len(seg_seq) - seq_seg0[-1])
+        k, b = len(seg_seq), len(seq_seg0)
+        flat = torch.tensor(seg_seq + seg_t0 + seg_n + seq_seg0 + seq_nseg, dtype=torch.int32).to(ctx.device)
+        return {"seg_seq": flat[:k], "seg_t0": flat[k:2 * k], "seg_n": flat[2 * k:3 * k], "seq_seg0": flat[3 * k:3 * k + b],
+                "seq_nseg": flat[3 * k + b:], "n": k}
+    return ctx.shared(("ssm_segments", length), make)
+
+
+def ssm_scan(xbc, proj, dt_col, dt_bias, a_log, d_skip, state, ctx, heads, groups, n_state, dv, segments=None) -> torch.Tensor:
+    """The selective state-space recurrence in float32.  ``xbc`` float32 [T, heads * dv + 2 groups n_state] (x | B |
+    C), the raw step sizes in ``proj`` columns dt_col .. dt_col + heads; ``state`` float32 [slots, heads, n_state,
+    dv], read and left up to date; returns y float32 [T, heads * dv].  ``segments`` (``ssm_segments``): the tokens
+    run in segments side by side, each twice (first for what it adds to the state, then, from the state before it,
+    for y); None: every sequence token by token in order."""
     _dev(xbc, proj, dt_bias, a_log, d_skip, state)
     _f32_rows(xbc, "ssm x/B/C")
     _f32_rows(proj, "ssm projections")
@@ -1258,6 +1349,19 @@ def ssm_scan(xbc, proj, dt_col, dt_bias, a_log, d_skip, state, ctx, heads, group
     qstart, qlen = getattr(ctx, "seq_qstart", None), getattr(ctx, "seq_qlen", None)
     _need((qstart is None) == (qlen is None) and (qstart is not None or t == ctx.n_seqs), "ssm: per-sequence starts and lengths")
     y = torch.empty((t, heads * dv), dtype=torch.float32, device=xbc.device)
+    if segments is not None:
+        _need(qstart is not None, "ssm in segments: per-sequence starts and lengths")
+        k = segments["n"]
+        for name, n in (("seg_seq", k), ("seg_t0", k), ("seg_n", k), ("seq_seg0", ctx.n_seqs), ("seq_nseg", ctx.n_seqs)):
+            _i32(segments[name], n, "ssm " + name)
+        seg_state = torch.empty((k, heads, n_state, dv), dtype=torch.float32, device=xbc.device)
+        seg_decay = torch.empty((k, heads), dtype=torch.float32, device=xbc.device)
+        _check(hybrid().li_ssm_scan_segments(
+            _ptr(xbc), xbc.shape[1], _ptr(proj), proj.shape[1], dt_col, _ptr(dt_bias), _ptr(a_log), _ptr(d_skip), _ptr(state),
+            _ptr(ctx.seq_slot), _ptr(qstart), _ptr(qlen), _ptr(y), ctx.n_seqs, heads, groups, n_state, dv,
+            _ptr(segments["seg_seq"]), _ptr(segments["seg_t0"]), _ptr(segments["seg_n"]), _ptr(segments["seq_seg0"]),
+            _ptr(segments["seq_nseg"]), k, _ptr(seg_state), _ptr(seg_decay), _stream()), "ssm_scan_segments")
+        return y
     _check(hybrid().li_ssm_scan(_ptr(xbc), xbc.shape[1], _ptr(proj), proj.shape[1], dt_col, _ptr(dt_bias), _ptr(a_log),
                                 _ptr(d_skip), _ptr(state), _ptr(ctx.seq_slot), _ptr(qstart), _ptr(qlen), _ptr(y), ctx.n_seqs,
                                 heads, groups, n_state, dv, _stream()), "ssm_scan")
@@ -1307,6 +1411,42 @@ def scale_blocks(t, weights, n_blocks, ff, tail) -> torch.Tensor:
     _need(weights.dtype == torch.float32 and weights.shape == (t.shape[0], n_blocks + int(tail > 0)), "scale_blocks: a weight for every block")
     _check(hybrid().li_scale_blocks(_ptr(t), DT[t.dtype], _ptr(weights), t.shape[0], n_blocks, ff, tail, _stream()), "scale_blocks")
     return t
+
+
+def moe_buckets(weights, n_experts: int):
+    """For each of the first ``n_experts`` columns of ``weights`` (float32 [T, cols]) the tokens whose weight is
+    not zero, ascending: int32 [n_experts, T] on the device and the counts as a list.  Waits for the device."""
+    _dev(weights)
+    _need(weights.dtype == torch.float32 and weights.dim() == 2 and weights.shape[1] >= n_experts, "moe_buckets: float32 [T, >= experts]")
+    t = weights.shape[0]
+    idx = torch.empty((n_experts, t), dtype=torch.int32, device=weights.device)
+    counts = torch.empty((n_experts,), dtype=torch.int32, device=weights.device)
+    _check(hybrid().li_moe_buckets(_ptr(weights), weights.shape[1], t, n_experts, _ptr(idx), _ptr(counts), _stream()), "moe_buckets")
+    return idx, counts.tolist()
+
+
+def gather_rows(h, idx, n: int) -> torch.Tensor:
+    """out[r] = h[idx[r]] for the first ``n`` entries of ``idx`` (int32, contiguous)."""
+    _dev(h, idx)
+    _need(h.dim() == 2 and h.dtype in DT and idx.dtype == torch.int32 and idx.numel() >= n, "gather_rows: rows and int32 indices")
+    out = torch.empty((n, h.shape[1]), dtype=h.dtype, device=h.device)
+    _check(hybrid().li_gather_rows(_ptr(h), DT[h.dtype], _ptr(idx), _ptr(out), n, h.shape[1], _stream()), "gather_rows")
+    return out
+
+
+def scatter_add_rows(residual, y, idx, weights, col: int) -> None:
+    """residual[idx[r]] += weights[idx[r]][col] * y[r] for every row of ``y`` (``idx`` None: row r itself); no row
+    may be named twice."""
+    _dev(residual, y, idx, weights)
+    n, width = y.shape
+    _need(residual.dtype == torch.float32 and y.dtype == torch.float32 and residual.shape[1] == width, "scatter_add_rows: float32 rows of one width")
+    _need(weights.dtype == torch.float32 and weights.dim() == 2 and weights.shape[0] == residual.shape[0] and 0 <= col < weights.shape[1],
+          "scatter_add_rows: a weight for every row of the residual")
+    _need(idx is None and n == residual.shape[0] or idx is not None and idx.dtype == torch.int32 and idx.numel() >= n,
+          "scatter_add_rows: int32 indices for every row of y")
+    _drop_row_stats(residual)
+    _check(hybrid().li_scatter_add_rows(_ptr(residual), _ptr(y), _ptr(idx), _ptr(weights), weights.shape[1], col, n, width,
+                                        _stream()), "scatter_add_rows")
 
 
 def copy_rows(x: torch.Tensor) -> torch.Tensor:

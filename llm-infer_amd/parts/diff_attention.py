@@ -33,7 +33,10 @@ class DifferentialAttention(Part):
     Scores, weights and all norms are float32 whatever the matrices' type.
 
     The three input projections are one product against [Wq; Wk; Wv].  The cache keeps, for every token, the
-    normed keys of all maps side by side and the values; pages behind the newest token's block are given back.
+    normed keys of all maps side by side (each padded to a multiple of 16) and the values, in the matrix cores'
+    operand order; pages behind the newest token's block are given back.  A 16-bit model runs prompts and decode
+    steps through one matrix-core kernel, compiled for the pair of head sizes at first use; a float32 model runs
+    one workgroup per (token, head).
     ``names``: local tensor names."""
 
     takes_lazy_norm = True
@@ -88,7 +91,8 @@ class DifferentialAttention(Part):
             self.lam = f32(f32(math.exp(dot("lq1", "lk1"))) - f32(math.exp(dot("lq2", "lk2"))) + self.lambda_init)
 
     def cache_spec(self):
-        return KVSpec(self.n_kv_heads, self.maps * self.head_dim, self.window, self.v_head_dim, self.block, "maps")
+        return KVSpec(self.n_kv_heads, self.maps * ops.padded_map_dim(self.head_dim), self.window, self.v_head_dim, self.block,
+                      "maps")
 
     def forward(self, h, ctx, view, residual, owns_cache=True):
         if not owns_cache:
@@ -98,5 +102,6 @@ class DifferentialAttention(Part):
         kv = view.as_tuple()
         q = ops.qk_norm_store(proj, 0, self.q_norm, self.k_norm, self.qk_norm_eps, ctx.pos, ctx.tok_slot, kv, H, G, m, d, dv)
         a = ops.diff_attention(q, kv, ctx.pos, ctx.tok_slot, H, G, m, d, dv, self.scale, self.block, self.window, self.lam,
-                               self.out_norm_eps, self.out_scale, self.dtype)
+                               self.out_norm_eps, self.out_scale, self.dtype,
+                               ops.diff_tiles(ctx) if self.dtype != torch.float32 else None)
         ops.linear(a, self.wo, ops.EPI_ADD, out=residual)

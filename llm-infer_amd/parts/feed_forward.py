@@ -4,6 +4,7 @@ import torch
 
 from ..kernels import ops
 from ..registry import register_feed_forward
+from ..tensor import Tensor
 from ..weights.loader import ParamSpec
 from .base import Part
 
@@ -118,12 +119,17 @@ class RoutedExperts(Part):
     ``shared_ff`` > 0: one more expert of that width runs for every token; ``shared_gate``: it is weighted by
     sigmoid(w_sg . h).
 
-    How it runs: the experts' gate and up matrices are stacked (the shared expert's behind them) into one
-    product whose epilogue applies silu(gate) * up; every expert's block of the hidden row is multiplied by the
-    token's weight for that expert, zero where it was not chosen; one product against the down matrices side by
-    side then sums the experts.  Every token so runs through every expert's matrices: the same numbers as
-    running only the chosen ones, no sorting of tokens, no shapes that depend on the data (a step can be
-    recorded), at n_experts / top times the arithmetic."""
+    How it runs.  Few tokens (a decode step, a short prompt, and every step of a float32 model): the experts' gate
+    and up matrices are stacked (the shared expert's behind them) into one product whose epilogue applies
+    silu(gate) * up; every expert's block of the hidden row is multiplied by the token's weight for that expert,
+    zero where it was not chosen; one product against the down matrices side by side then sums the experts.
+    Every token so runs through every expert's matrices: the same numbers as running only the chosen ones, every
+    matrix streamed once, no shapes that depend on the data (a step can be recorded), at n_experts / top times the
+    arithmetic.  Many tokens in a 16-bit model (``GROUPED_FROM`` rows an expert on average): the tokens are listed
+    by expert on the device, the host reads the eight or so counts, and every expert runs its own two products on
+    its own tokens' rows, added into the residual rows expert by expert (a fixed order)."""
+
+    GROUPED_FROM = 48
 
     def __init__(self, *, hidden_size, n_experts, expert_ff, top, n_identity=0, route_scale=1.0, correction=True,
                  shared_ff=0, shared_gate=True, names=None, prefix, dtype, device):
@@ -162,14 +168,48 @@ class RoutedExperts(Part):
             down.append(tensors[p + n["down"]])
         self.w_gate_up = ops.prepare_weight(torch.cat(gu, 0).contiguous())
         self.w_down = ops.prepare_weight(torch.cat(down, 1).contiguous())
+        # for prompts: every expert's matrices by themselves (gate and up as row ranges of the stacked matrix where
+        # its tiles allow, the down matrices as copies of their own)
+        self.per_expert = None
+        if self.dtype != torch.float32:
+            parts, at = [], 0
+            for (p, f), g_u, d_ in zip(self._experts(), gu, down):
+                parts.append((self._rows(self.w_gate_up, at, 2 * f, g_u), ops.prepare_weight(d_.contiguous())))
+                at += 2 * f
+            self.per_expert = parts
         rows = [tensors[n["router"]].float()] + ([tensors[n["shared_gate"]].float().view(1, d)] if self.shared_gate else [])
-        self.w_router = ops.prepare_weight(torch.cat(rows, 0).contiguous())   # float32: the logits are summed in float32
+        self.w_router = torch.cat(rows, 0).contiguous()                       # float32: the logits are summed in float32
         self.bias = tensors[n["correction"]] if self.correction else None
 
+    @staticmethod
+    def _rows(stacked, r0, n, own):
+        """Rows r0 .. r0 + n of a stacked matrix as a matrix of its own, sharing the storage where the tiled layout
+        allows (ranges that begin and end at multiples of 16 rows); else a copy."""
+        if ops.is_tiled(stacked) and r0 % 16 == 0 and n % 16 == 0:
+            k = ops.matrix_shape(stacked)[1]
+            flat = stacked.as_subclass(torch.Tensor)[r0 * k:(r0 + n) * k]
+            return Tensor.wrap(flat, "tiled", (n, k), stacked.owner, stacked)
+        return ops.prepare_weight(own.contiguous())
+
+    def _grouped(self, h, residual, weights):
+        idx, counts = ops.moe_buckets(weights, self.n_experts)
+        for e, n in enumerate(counts):
+            if n:
+                w_gu, w_d = self.per_expert[e]
+                t = ops.linear(ops.gather_rows(h, idx[e], n), w_gu, ops.EPI_SWIGLU, out_dtype=self.dtype)
+                ops.scatter_add_rows(residual, ops.linear(t, w_d, out_dtype=torch.float32), idx[e], weights, e)
+        if self.shared_ff:
+            w_gu, w_d = self.per_expert[self.n_experts]
+            t = ops.linear(h, w_gu, ops.EPI_SWIGLU, out_dtype=self.dtype)
+            ops.scatter_add_rows(residual, ops.linear(t, w_d, out_dtype=torch.float32), None, weights, self.n_experts)
+
     def forward(self, h, residual):
-        logits = ops.linear(h, self.w_router, out_dtype=torch.float32)
+        logits = ops.small_logits(h, self.w_router)
         weights = ops.moe_route(logits, self.bias, h, residual, self.n_experts + self.n_identity, self.n_experts, self.top,
                                 (1 if self.shared_gate else 2) if self.shared_ff else 0, self.route_scale)
+        if (self.per_expert is not None and self.n_experts and h.shape[0] * self.top >= self.GROUPED_FROM * self.n_experts
+                and not torch.cuda.is_current_stream_capturing()):
+            return self._grouped(h, residual, weights)
         t = ops.linear(h, self.w_gate_up, ops.EPI_SWIGLU, out_dtype=self.dtype)
         ops.scale_blocks(t, weights, self.n_experts, self.expert_ff, self.shared_ff)
         ops.linear(t, self.w_down, ops.EPI_ADD, out=residual)

@@ -74,7 +74,12 @@ class SelectiveStateSpace(Part):
         state, history = views[0].state, views[1].state
         proj = ops.linear(h, self.w_in, out_dtype=torch.float32)
         xbc = ops.conv_silu(proj, self.inner, self.channels, self.conv, self.conv_bias, history, ctx)
+        # a 16-bit model walks long prompts in segments side by side; a float32 model (and every decode step) walks each
+        # sequence in order, which gives the same bits however a prompt is cut
+        segments = None
+        if self.dtype != torch.float32 and not ctx.is_decode and max(getattr(ctx, "host_qlens", None) or [0]) > ops.SSM_SEGMENT:
+            segments = ops.ssm_segments(ctx)
         y = ops.ssm_scan(xbc, proj, self.inner + self.channels, self.dt_bias, self.a_log, self.d_skip, state, ctx,
-                         self.n_heads, self.n_groups, self.n_state, self.head_dim)
+                         self.n_heads, self.n_groups, self.n_state, self.head_dim, segments)
         a = ops.gated_group_norm(y, proj, 0, self.norm, self.norm_groups, self.norm_eps, self.dtype)
         ops.linear(a, self.wo, ops.EPI_ADD, out=residual)

@@ -81,15 +81,18 @@ def diff_lambda(t, diff):
     return torch.exp((t["lq1"] * t["lk1"]).sum()) - torch.exp((t["lq2"] * t["lk2"]).sum()) + diff
 
 
-def diff_attention(h, t, m, eps):
-    """``t``: the mixer's tensors by local name (q, k, v, o, q.norm, k.norm, lq1, lk1, lq2, lk2); ``m``: its sizes."""
+def diff_attention(h, t, m, eps, store=None):
+    """``t``: the mixer's tensors by local name (q, k, v, o, q.norm, k.norm, lq1, lk1, lq2, lk2); ``m``: its sizes.
+    ``store`` (a 16-bit type): q, k, v and the heads' outputs take that type's values where a 16-bit engine stores
+    them, which measures what that rounding alone does to the result."""
     H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
     n = h.shape[0]
-    q = rms_div((h @ t["q"].T).view(n, H, 2, d), eps) * t["q.norm"]
-    k = rms_div((h @ t["k"].T).view(n, G, 2, d), eps) * t["k.norm"]
-    v = (h @ t["v"].T).view(n, G, dv)
+    r = (lambda x: x.to(store).to(x.dtype)) if store is not None else (lambda x: x)
+    q = r(rms_div((h @ t["q"].T).view(n, H, 2, d), eps) * t["q.norm"])
+    k = r(rms_div((h @ t["k"].T).view(n, G, 2, d), eps) * t["k.norm"])
+    v = r((h @ t["v"].T).view(n, G, dv))
     out = diff_attention_core(q, k, v, m["scale"], diff_lambda(t, m["diff"]), int(m["mask"]["size"]), eps, 1.0 - m["diff"])
-    return out.reshape(n, H * dv) @ t["o"].T
+    return r(out.reshape(n, H * dv)) @ t["o"].T
 
 
 # ------------------------------------------------------------------ the state-space mixer

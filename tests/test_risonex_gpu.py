@@ -59,6 +59,7 @@ def error(got, ref):
 
 def build_part(table, spec, weights, dtype):
     """A part as the configuration describes it, with the given tensors (by local name) bound."""
+    import llm_infer_amd.parts  # noqa: F401  (registers the parts)
     from llm_infer_amd.registry import lookup
     from llm_infer_amd.weights.loader import place_tensor
     extra = {"position": None} if table == "mixer" else {}
@@ -175,14 +176,17 @@ def test_differential_attention_part(lib, dtype, H, G, d, dv, block, schedule):
     mixer = M.attention(H, G, d, dv, block, diff=0.3)
     cfg = one_layer(mixer, width=width, eps=eps)
     g = torch.Generator().manual_seed(H * 100 + d)
-    W = M.mixer_weights("attention", mixer[1], width, g, torch.bfloat16, sharp=3.0)
+    W = M.mixer_weights("attention", mixer[1], width, g, torch.bfloat16, sharp=2.0)
     part = build_part("mixer", cfg._mixer("", cfg.layers[0]), W, dtype)
     n = {"a": 140, "b": 9, "c": 70}
     h_of = {r: torch.randn(k, width, generator=g).to(DT[dtype]).float() for r, k in n.items()}
     got, cache = run_mixer(part, h_of, SCHEDULES[schedule](n), dtype)
     for r in n:
         ref = P.diff_attention(h_of[r].double(), M.widen(W), mixer[1], eps)
-        assert error(got[r], ref) < TOL[dtype], r
+        tol = TOL[dtype]
+        if dtype == "bfloat16":      # not below three times what the rounding of q, k, v and the output alone does
+            tol = max(tol, 3 * error(P.diff_attention(h_of[r].double(), M.widen(W), mixer[1], eps, store=torch.bfloat16), ref))
+        assert error(got[r], ref) < tol, r
     assert all(g_.pool.n_free == g_.n_pages - 1 for g_ in cache.groups)         # every page came back
 
 
@@ -198,13 +202,13 @@ def test_attention_sees_its_block_and_nothing_before_it(lib, dtype):
     g = torch.Generator().manual_seed(9)
     H, G, d, dv, T, B = 2, 1, 32, 48, 420, 150
     q, k, v = torch.randn(T, H, 2, d, generator=g), torch.randn(T, G, 2, d, generator=g), torch.randn(T, G, dv, generator=g)
-    if dtype == "bfloat16":
-        k, v = k.bfloat16().float(), v.bfloat16().float()
     probes = (149, 150, 151, 299, 300, 310, 419)
     for t in probes:
         lo = t - t % B
         q[t, :, 0] = k[lo, 0, 0] * 4.0
         q[t, :, 1] = k[max(lo - 1, 0), 0, 1] * 4.0
+    if dtype == "bfloat16":                      # what the cache and the kernel's q hold
+        q, k, v = q.bfloat16().float(), k.bfloat16().float(), v.bfloat16().float()
     lam, scale = 0.6, 1.0
     ref = P.diff_attention_core(q.double(), k.double(), v.double(), scale, lam, B, 1e-6, 0.7)
     # the same tokens one position later (a token put in front): every block then begins one token earlier, which is
@@ -222,7 +226,8 @@ def test_attention_sees_its_block_and_nothing_before_it(lib, dtype):
         qkv = torch.cat([q[rows].reshape(n, -1), k[rows].reshape(n, -1), v[rows].reshape(n, -1)], 1).to(DEV)
         kv = cache.view(0).as_tuple()
         qd = ops.qk_norm_store(qkv, 0, None, None, None, ctx.pos, ctx.tok_slot, kv, H, G, 2, d, dv)
-        out = ops.diff_attention(qd, kv, ctx.pos, ctx.tok_slot, H, G, 2, d, dv, scale, B, None, lam, 1e-6, 0.7, dt)
+        out = ops.diff_attention(qd, kv, ctx.pos, ctx.tok_slot, H, G, 2, d, dv, scale, B, None, lam, 1e-6, 0.7, dt,
+                                 ops.diff_tiles(ctx) if dtype != "float32" else None)
         got.append(out.cpu().double().view(n, H, dv))
         at += n
         cache.trim_windows([slot])
@@ -324,6 +329,37 @@ def test_feed_forward_parts(lib, dtype, mlp):
         alone = torch.zeros(1, width, device=DEV)                          # a token's rows do not depend on the batch
         part.forward(h[-1:].to(DEV), alone)
         assert error(alone.cpu(), ref[-1:]) < TOL[dtype]
+
+
+def test_routed_experts_sorted_by_expert_in_a_long_prompt(lib):
+    """A bfloat16 prompt long enough that the tokens are listed by expert and every expert runs on its own rows,
+    with a choice that differs from token to token and margins that no rounding can turn: a token's input has a
+    large entry where its first expert's router row has its only weight and a smaller one for its second."""
+    width, mlp = 96, M.moe(4, 2, 48, identity=1, scale=1.3, shared=32)
+    cfg = one_layer(M.mamba(2, 8, 8), mlp, width=width)
+    g = torch.Generator().manual_seed(17)
+    W = M.mlp_weights(mlp, width, g, torch.bfloat16)
+    W["router"] = torch.zeros(5, width, dtype=torch.bfloat16)
+    W["router"][torch.arange(5), torch.arange(5)] = 2.0
+    W["correction"] = torch.zeros(5, dtype=torch.bfloat16)
+    part = build_part("feed_forward", cfg._feed_forward("", mlp), W, "bfloat16")
+    T = 400
+    assert T * 2 >= part.GROUPED_FROM * 4 and part.per_expert is not None
+    h = 0.3 * torch.randn(T, width, generator=g)
+    first = torch.randint(0, 5, (T,), generator=g)
+    second = (first + torch.randint(1, 5, (T,), generator=g)) % 5
+    h[torch.arange(T), first] += 4.0
+    h[torch.arange(T), second] += 2.0
+    h = h.bfloat16()
+    chosen, _ = P.route(h.double(), M.widen(W), mlp["router"])
+    assert torch.equal(chosen.sort(-1).values, torch.stack([first, second], 1).sort(-1).values)
+    res = torch.zeros(T, width, device=DEV)
+    part.forward(h.to(DEV), res)
+    ref = P.moe_ff(h.double(), M.widen(W), mlp)
+    assert error(res.cpu(), ref) < TOL["bfloat16"]
+    few = torch.zeros(7, width, device=DEV)                      # the same rows among few: every token through every expert
+    part.forward(h[:7].to(DEV), few)
+    assert error(few.cpu(), ref[:7]) < TOL["bfloat16"]
 
 
 def test_reinject_multiplies_stream_and_embedding_side_by_side(lib):
