@@ -3,7 +3,8 @@
 // values and queries; scores, weights, sums and the norm of the output float32.
 //
 // One wave per (tile of up to 32 consecutive tokens of a sequence, query head); a decode step's tiles hold one
-// token.  A token at position p sees the keys lo .. p, lo = p - p % block (block 0: 0; window w: at least p - w + 1).
+// token, and four waves then take every fourth 32 keys each and merge their running maxima, sums and outputs
+// through LDS in wave order.  A token at position p sees the keys lo .. p, lo = p - p % block (block 0: 0; window w: at least p - w + 1).
 // Keys are walked 32 at a time.  Per map m:  S^T = K_m Q_m^T  (rows keys, columns queries; operand A straight from
 // the page, which holds keys in operand order), online softmax down the rows (a query's 32 scores lie in the 16
 // accumulator elements of two lanes), then O_m^T += V^T P_m^T with the accumulators' own order of the keys, in which the
@@ -27,13 +28,19 @@ struct MapPages {
 };
 
 template <class T, int MAPS>
-__global__ __launch_bounds__(64) void diff_attn_mfma_kernel(
+__global__ __launch_bounds__(256) void diff_attn_mfma_kernel(
     const T* __restrict__ q, T* __restrict__ out, MapPages pg, const int* __restrict__ pos,
     const int* __restrict__ tok_slot, const int* __restrict__ tile_t0, const int* __restrict__ tile_n, int H, int G,
-    int dv, float scale, int block, int window, float lambda, float out_eps, float out_scale) {
+    int dv, float scale, int block, int window, float lambda, float out_eps, float out_scale, int split) {
     typedef typename Vec<T>::v8 v8;
     constexpr int D16 = MAP_DIM / 16, KW = MAPS * MAP_DIM, DVB = VALUE_DIM / 32;
-    const int tile = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, col = lane & 31, half = lane >> 5;
+    extern __shared__ float lds[];
+    const int tile = blockIdx.x, lane = threadIdx.x & 63, col = lane & 31, half = lane >> 5;
+    const int wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    // the waves of a workgroup: the query heads of one KV head on the same tile (they fetch the same keys and
+    // values, which then come from the CU's cache), or, `split`, shares of the keys of a tile of one token
+    const int h = split ? blockIdx.y : blockIdx.y * nw + wave;
+    const int kwave = split ? wave : 0, kstep = split ? nw : 1;
     const int t0 = tile_t0 ? tile_t0[tile] : tile, n = tile_n ? tile_n[tile] : 1;
     if (n <= 0) return;
     const int g = h / (H / G);
@@ -81,9 +88,9 @@ __global__ __launch_bounds__(64) void diff_attn_mfma_kernel(
 #pragma unroll
             for (int u = 0; u < 2; ++u) vn[b][u] = *(const v8*)(vh + ((int64_t)(b * (PAGE / 16) + tb * 2 + u) * 64 + lane) * 8);
     };
-    const int kt_last = p_last / 32;
-    fetch(lo_tile / 32);
-    for (int kt = lo_tile / 32; kt <= kt_last; ++kt) {
+    const int kt_last = p_last / 32, kt_first = lo_tile / 32 + kwave;
+    if (kt_first <= kt_last) fetch(kt_first);
+    for (int kt = kt_first; kt <= kt_last; kt += kstep) {
         v8 kf[MAPS][D16], vf[DVB][2];
 #pragma unroll
         for (int a = 0; a < MAPS; ++a)
@@ -93,7 +100,7 @@ __global__ __launch_bounds__(64) void diff_attn_mfma_kernel(
         for (int b = 0; b < DVB; ++b)
 #pragma unroll
             for (int u = 0; u < 2; ++u) vf[b][u] = vn[b][u];
-        if (kt < kt_last) fetch(kt + 1);
+        if (kt + kstep <= kt_last) fetch(kt + kstep);
         v8 phi[MAPS][2], plo[MAPS][2];
 #pragma unroll
         for (int a = 0; a < MAPS; ++a) {
@@ -153,6 +160,46 @@ __global__ __launch_bounds__(64) void diff_attn_mfma_kernel(
                 }
             }
     }
+    if (split && nw > 1) {
+        // a tile of one token whose keys the waves have shared: wave 0 adds up their states in wave order
+        constexpr int W = 2 + VALUE_DIM;
+        if (col == 0) {
+#pragma unroll
+            for (int a = 0; a < MAPS; ++a) {
+                float* mine = lds + (wave * MAPS + a) * W;
+                if (half == 0) { mine[0] = m[a]; mine[1] = l[a]; }
+#pragma unroll
+                for (int b = 0; b < DVB; ++b)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) mine[2 + b * 32 + 8 * (r >> 2) + 4 * half + (r & 3)] = o[a][b][r];
+            }
+        }
+        __syncthreads();
+        if (wave != 0) return;
+        if (col == 0) {
+#pragma unroll
+            for (int a = 0; a < MAPS; ++a) {
+                float M = -INFINITY;
+                for (int w = 0; w < nw; ++w) M = fmaxf(M, lds[(w * MAPS + a) * W]);
+                float L = 0.f;
+#pragma unroll
+                for (int b = 0; b < DVB; ++b)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) o[a][b][r] = 0.f;
+                for (int w = 0; w < nw; ++w) {
+                    const float* theirs = lds + (w * MAPS + a) * W;
+                    if (theirs[0] == -INFINITY) continue;
+                    const float f = expf(theirs[0] - M);
+                    L += theirs[1] * f;
+#pragma unroll
+                    for (int b = 0; b < DVB; ++b)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) o[a][b][r] += theirs[2 + b * 32 + 8 * (r >> 2) + 4 * half + (r & 3)] * f;
+                }
+                m[a] = M; l[a] = L;
+            }
+        }
+    }
     // o = O_1 / l_1 - lambda O_2 / l_2 for this lane's query; its values lie in this lane and in lane ^ 32
     float ss = 0.f;
 #pragma unroll
@@ -194,9 +241,15 @@ extern "C" int li_diffattn(const void* q, void* out, int dt, const void* k_pages
     if (maps < 1 || maps > 2 || (dt != DT_F16 && dt != DT_BF16)) return LI_UNSUPPORTED;
     if ((tile_t0 == nullptr) != (tile_n == nullptr)) return LI_BAD_ARG;
     MapPages pg{k_pages, v_pages, page_stride, page_table, max_pages};
-    dim3 grid(n_tiles, H);
-#define GO(T, M) diff_attn_mfma_kernel<T, M><<<grid, 64, 0, stream>>>((const T*)q, (T*)out, pg, pos, tok_slot, tile_t0, tile_n, \
-                                                                      H, G, dv, scale, block, window, lambda, out_eps, out_scale)
+    // tiles of one token (a decode step): four waves share a token's keys and merge through LDS; else the waves of
+    // a workgroup are query heads of one KV head (4, 2 or 1 of them)
+    const int split = tile_t0 ? 0 : 1, per_kv = H / G;
+    const int heads = split ? 1 : (per_kv % 4 == 0 ? 4 : (per_kv % 2 == 0 ? 2 : 1));
+    dim3 grid(n_tiles, H / heads);
+    const int threads = split ? 256 : 64 * heads;
+    const size_t lds = split ? (size_t)4 * maps * (2 + VALUE_DIM) * sizeof(float) : 0;
+#define GO(T, M) diff_attn_mfma_kernel<T, M><<<grid, threads, lds, stream>>>((const T*)q, (T*)out, pg, pos, tok_slot, tile_t0, tile_n, \
+                                                                      H, G, dv, scale, block, window, lambda, out_eps, out_scale, split)
     if (dt == DT_F16) { if (maps == 1) GO(f16, 1); else GO(f16, 2); }
     else { if (maps == 1) GO(bf16, 1); else GO(bf16, 2); }
 #undef GO

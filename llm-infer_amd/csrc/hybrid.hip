@@ -117,8 +117,8 @@ __global__ void qk_norm_store_kernel(const float* __restrict__ qkv, int stride, 
     const int page = pg.page_table[(int64_t)tok_slot[t] * pg.max_pages + p / PAGE], off = p % PAGE;
     T* kp = (T*)pg.k + (int64_t)page * pg.page_stride;
     T* vp = (T*)pg.v + (int64_t)page * pg.page_stride;
-    const int n_units = (H + G) * maps;                   // one wave a (head, map)
-    for (int u = wave; u < n_units; u += nw) {
+    const int n_units = (H + G) * maps;                   // one wave a (head, map), the units over the grid's second dimension
+    for (int u = blockIdx.y * nw + wave; u < n_units; u += gridDim.y * nw) {
         const bool is_q = u < H * maps;
         const float* src = row + (int64_t)u * d;          // q heads then k heads, each maps * d wide
         float ss = 0.f;
@@ -135,7 +135,7 @@ __global__ void qk_norm_store_kernel(const float* __restrict__ qkv, int stride, 
         }
     }
     const float* vsrc = row + (int64_t)(H + G) * maps * d;
-    for (int i = threadIdx.x; i < G * dv; i += blockDim.x) {
+    for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < G * dv; i += gridDim.y * blockDim.x) {
         const int g = i / dv, j = i - g * dv;
         vp[g * v_head_elems(dv) + v_offset(off, j, dv)] = from_f32<T>(vsrc[i]);
     }
@@ -148,7 +148,8 @@ extern "C" int li_qk_norm_store(const float* qkv, int stride, int col0, const fl
     if (n <= 0) return LI_OK;
     if (H <= 0 || G <= 0 || maps <= 0 || d <= 0 || dv <= 0) return LI_BAD_ARG;
     MapPages pg{k_pages, v_pages, page_stride, page_table, max_pages};
-    DISPATCH_T(dt, (qk_norm_store_kernel<T><<<n, 256, 0, stream>>>(qkv, stride, col0, qw, kw, eps, pos, tok_slot, (T*)q_out,
+    dim3 grid(n, n >= 512 ? 1 : ((H + G) * maps + 3) / 4);       // few tokens: a wave for every (head, map)
+    DISPATCH_T(dt, (qk_norm_store_kernel<T><<<grid, 256, 0, stream>>>(qkv, stride, col0, qw, kw, eps, pos, tok_slot, (T*)q_out,
                                                                   pg, H, G, maps, d, dv)));
     LI_CHECK_LAUNCH();
     return LI_OK;
@@ -571,17 +572,19 @@ __global__ __launch_bounds__(64) void small_logits_kernel(const T* __restrict__ 
     const int t = blockIdx.x, j = blockIdx.y, lane = threadIdx.x;
     const T* row = h + (int64_t)t * width;
     const float* wj = w + (int64_t)j * width;
-    float part[8];
+    float part[16];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) part[u] = 0.f;
-    for (int i0 = 0; i0 < width; i0 += 512) {              // eight independent loads of each operand at a time
+    for (int u = 0; u < 16; ++u) part[u] = 0.f;
+    for (int i0 = 0; i0 < width; i0 += 1024) {             // sixteen independent loads of each operand at a time
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
+        for (int u = 0; u < 16; ++u) {
             const int i = i0 + u * 64 + lane;
             if (i < width) part[u] += wj[i] * to_f32(row[i]);
         }
     }
-    float acc = ((part[0] + part[1]) + (part[2] + part[3])) + ((part[4] + part[5]) + (part[6] + part[7]));
+    float acc = 0.f;
+#pragma unroll
+    for (int u = 0; u < 16; ++u) acc += part[u];
     acc = wave_sum(acc);
     if (lane == 0) out[(int64_t)t * n + j] = acc;
 }

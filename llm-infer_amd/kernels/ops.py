@@ -1305,7 +1305,8 @@ def conv_silu(rows, col0, channels, weight, bias, history, ctx) -> torch.Tensor:
     return out
 
 
-SSM_SEGMENT = 128          # tokens of a segment when a prompt's recurrence runs in segments side by side
+SSM_SEGMENT = 128          # most tokens of a segment when a prompt's recurrence runs in segments side by side
+SSM_WAVES = 3072           # segments are made short enough for about this many waves (three a SIMD)
 
 
 def ssm_segments(ctx, length: int | None = None) -> dict:

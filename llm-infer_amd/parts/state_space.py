@@ -77,8 +77,12 @@ class SelectiveStateSpace(Part):
         # a 16-bit model walks long prompts in segments side by side; a float32 model (and every decode step) walks each
         # sequence in order, which gives the same bits however a prompt is cut
         segments = None
-        if self.dtype != torch.float32 and not ctx.is_decode and max(getattr(ctx, "host_qlens", None) or [0]) > ops.SSM_SEGMENT:
-            segments = ops.ssm_segments(ctx)
+        if self.dtype != torch.float32 and not ctx.is_decode and getattr(ctx, "host_qlens", None):
+            # segments short enough that some 3,000 waves run (three a SIMD), between 16 and SSM_SEGMENT tokens
+            waves_a_token = self.n_heads * ((self.head_dim + 63) // 64)
+            length = max(16, min(ops.SSM_SEGMENT, 1 << max(0, (ctx.n_tokens * waves_a_token // ops.SSM_WAVES).bit_length() - 1)))
+            if max(ctx.host_qlens) > length:
+                segments = ops.ssm_segments(ctx, length)
         y = ops.ssm_scan(xbc, proj, self.inner + self.channels, self.dt_bias, self.a_log, self.d_skip, state, ctx,
                          self.n_heads, self.n_groups, self.n_state, self.head_dim, segments)
         a = ops.gated_group_norm(y, proj, 0, self.norm, self.norm_groups, self.norm_eps, self.dtype)
