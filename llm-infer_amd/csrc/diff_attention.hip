@@ -52,6 +52,10 @@ __global__ __launch_bounds__(256) void diff_attn_mfma_kernel(
     int lo_tile = block > 0 ? p0 - p0 % block : 0;     // the first token's: the smallest
     if (window > 0) lo_tile = max(lo_tile, p0 - window + 1);
     const int p_last = p0 + n - 1;
+    int lo_last = block > 0 ? p_last - p_last % block : 0;       // the last token's: the largest
+    if (window > 0) lo_last = max(lo_last, p_last - window + 1);
+    const bool whole_tile = n == 32;
+    const float scale2 = scale * 1.4426950408889634f;
     const int* table = pg.page_table + (int64_t)tok_slot[t0] * pg.max_pages;
 
     v8 qf[MAPS][D16];
@@ -111,13 +115,20 @@ __global__ __launch_bounds__(256) void diff_attn_mfma_kernel(
             for (int s = 0; s < D16; ++s) {
                 acc = mfma32(kf[a][s], qf[a][s], acc);
             }
+            // scores in units of log 2, so that a weight is one hardware 2^x; 32 keys that every query of a whole tile
+            // sees need no mask
             float tmax = -INFINITY;
+            if (whole_tile && kt * 32 >= lo_last && kt * 32 + 31 <= p0) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int key = kt * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-                const bool seen = has_query && key >= lo_q && key <= pq;
-                acc[r] = seen ? acc[r] * scale : -INFINITY;
-                tmax = fmaxf(tmax, acc[r]);
+                for (int r = 0; r < 16; ++r) { acc[r] *= scale2; tmax = fmaxf(tmax, acc[r]); }
+            } else {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int key = kt * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+                    const bool seen = has_query && key >= lo_q && key <= pq;
+                    acc[r] = seen ? acc[r] * scale2 : -INFINITY;
+                    tmax = fmaxf(tmax, acc[r]);
+                }
             }
             tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
             const float mn = fmaxf(m[a], tmax);
@@ -127,9 +138,9 @@ __global__ __launch_bounds__(256) void diff_attn_mfma_kernel(
 #pragma unroll
                 for (int r = 0; r < 16; ++r) pr[r] = 0.f;
             } else {
-                f = expf(m[a] - mn);                                       // 0 while m is still -inf
+                f = __builtin_amdgcn_exp2f(m[a] - mn);                     // 0 while m is still -inf
 #pragma unroll
-                for (int r = 0; r < 16; ++r) { pr[r] = expf(acc[r] - mn); sum += pr[r]; }
+                for (int r = 0; r < 16; ++r) { pr[r] = __builtin_amdgcn_exp2f(acc[r] - mn); sum += pr[r]; }
             }
             sum += __shfl_xor(sum, 32, WAVE);
             l[a] = l[a] * f + sum;
@@ -189,7 +200,7 @@ __global__ __launch_bounds__(256) void diff_attn_mfma_kernel(
                 for (int w = 0; w < nw; ++w) {
                     const float* theirs = lds + (w * MAPS + a) * W;
                     if (theirs[0] == -INFINITY) continue;
-                    const float f = expf(theirs[0] - M);
+                    const float f = __builtin_amdgcn_exp2f(theirs[0] - M);
                     L += theirs[1] * f;
 #pragma unroll
                     for (int b = 0; b < DVB; ++b)

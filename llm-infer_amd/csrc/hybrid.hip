@@ -2,8 +2,10 @@
 // a scaled embedding with sinusoidal positions, the per-head RMS norm of q and k with the write into the paged
 // cache, differential attention over blocks of positions (two softmax maps over the same values, combined and
 // normed per head), the short causal convolution with its per-sequence history, the selective state-space
-// recurrence with a float32 state per sequence, the gated norm in groups behind it, plain activations, the
-// router of a mixture of experts and the weighting of the experts' hidden rows.  Every size is a run-time value.
+// recurrence with a float32 state per sequence (token by token, or a prompt in segments side by side), the gated
+// norm in groups behind it, plain activations, the router of a mixture of experts (logits, choice, weights), the
+// weighting of the experts' hidden rows, and the lists of tokens by expert with the gather and scatter of their rows.
+// The 16-bit attention on the matrix cores is diff_attention.hip.  Every size is a run-time value.
 // Whatever a norm, a score, an attention weight, a decay, a step size or a recurrent state is made of is float32
 // here, whatever the type of the matrices.
 #include "common.h"
@@ -564,37 +566,52 @@ extern "C" int li_gated_group_norm(const float* y, const float* zrows, int z_str
 
 // ---------------------------------------------------------------------------
 // out[t][j] = w[j] . h[t] in float32 for a few rows of a float32 matrix w [n, width] (a router's): one
-// wave per (token, output), the lanes stride the width; every sum has one fixed order whatever the batch.
+// workgroup per (token, output), its threads stride the width; every sum has one fixed order whatever the batch.
 // ---------------------------------------------------------------------------
-template <class T>
-__global__ __launch_bounds__(64) void small_logits_kernel(const T* __restrict__ h, const float* __restrict__ w,
-                                                          float* __restrict__ out, int width, int n) {
-    const int t = blockIdx.x, j = blockIdx.y, lane = threadIdx.x;
-    const T* row = h + (int64_t)t * width;
+template <class T, int TOK>
+__global__ __launch_bounds__(256) void small_logits_kernel(const T* __restrict__ h, const float* __restrict__ w,
+                                                           float* __restrict__ out, int n_rows, int width, int n) {
+    __shared__ float scratch[16];
+    const int t0 = blockIdx.x * TOK, j = blockIdx.y, tid = threadIdx.x;
     const float* wj = w + (int64_t)j * width;
-    float part[16];
+    float part[TOK][16];
 #pragma unroll
-    for (int u = 0; u < 16; ++u) part[u] = 0.f;
-    for (int i0 = 0; i0 < width; i0 += 1024) {             // sixteen independent loads of each operand at a time
+    for (int k = 0; k < TOK; ++k)
+#pragma unroll
+        for (int u = 0; u < 16; ++u) part[k][u] = 0.f;
+    for (int i0 = 0; i0 < width; i0 += 4096) {             // sixteen independent loads of each operand a thread at a time
 #pragma unroll
         for (int u = 0; u < 16; ++u) {
-            const int i = i0 + u * 64 + lane;
-            if (i < width) part[u] += wj[i] * to_f32(row[i]);
+            const int i = i0 + u * 256 + tid;
+            if (i < width) {
+                const float wv = wj[i];                    // a weight is fetched once for the workgroup's TOK tokens
+#pragma unroll
+                for (int k = 0; k < TOK; ++k)
+                    if (t0 + k < n_rows) part[k][u] += wv * to_f32(h[(int64_t)(t0 + k) * width + i]);
+            }
         }
     }
-    float acc = 0.f;
 #pragma unroll
-    for (int u = 0; u < 16; ++u) acc += part[u];
-    acc = wave_sum(acc);
-    if (lane == 0) out[(int64_t)t * n + j] = acc;
+    for (int k = 0; k < TOK; ++k) {                        // the same order of sums for a token whatever TOK is
+        float acc = 0.f;
+#pragma unroll
+        for (int u = 0; u < 16; ++u) acc += part[k][u];
+        acc = block_sum(acc, scratch);                     // the waves' sums in wave order
+        if (tid == 0 && t0 + k < n_rows) out[(int64_t)(t0 + k) * n + j] = acc;
+    }
 }
 
 extern "C" int li_small_logits(const void* h, int dt, const float* w, float* out, int n_rows, int width, int n,
                                hipStream_t stream) {
     if (n_rows <= 0 || n <= 0) return LI_OK;
     if (width <= 0 || n > 65535) return LI_BAD_ARG;
-    dim3 grid(n_rows, n);
-    DISPATCH_T(dt, (small_logits_kernel<T><<<grid, 64, 0, stream>>>((const T*)h, w, out, width, n)));
+    if (n_rows >= 256) {                                   // many tokens: four a workgroup share every weight fetched
+        dim3 grid((n_rows + 3) / 4, n);
+        DISPATCH_T(dt, (small_logits_kernel<T, 4><<<grid, 256, 0, stream>>>((const T*)h, w, out, n_rows, width, n)));
+    } else {
+        dim3 grid(n_rows, n);
+        DISPATCH_T(dt, (small_logits_kernel<T, 1><<<grid, 256, 0, stream>>>((const T*)h, w, out, n_rows, width, n)));
+    }
     LI_CHECK_LAUNCH();
     return LI_OK;
 }

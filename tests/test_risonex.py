@@ -171,3 +171,19 @@ def test_the_cache_gives_back_the_pages_behind_a_block():
     assert sorted(blocked.pages_of[s]) == [4]
     cache.free_slot(s)
     assert blocked.pool.n_free == blocked.n_pages - 1
+
+
+def test_tiles_and_segments_are_planned_from_the_steps_lengths():
+    """The host's plans for a step: attention tiles of up to 32 consecutive tokens that never cross a sequence, and
+    the recurrence's segments with every sequence's first segment and count."""
+    from llm_infer_amd.engine.step import StepContext
+    from llm_infer_amd.kernels import ops
+    ctx = StepContext("cpu", [0, 1, 2], [[0] * 70, [0], [0] * 32], [5, 0, 100], [[], [], []])
+    t0, n, count = ops.diff_tiles(ctx)
+    assert count == 5 and t0.tolist() == [0, 32, 64, 70, 71] and n.tolist() == [32, 32, 6, 1, 32]
+    assert ops.diff_tiles(ctx) is ops.diff_tiles(ctx)                      # made once per step
+    seg = ops.ssm_segments(ctx, 32)
+    assert seg["n"] == 5 and seg["seg_seq"].tolist() == [0, 0, 0, 1, 2] and seg["seg_t0"].tolist() == [0, 32, 64, 0, 0]
+    assert seg["seg_n"].tolist() == [32, 32, 6, 1, 32] and seg["seq_seg0"].tolist() == [0, 3, 4] and seg["seq_nseg"].tolist() == [3, 1, 1]
+    decode = StepContext("cpu", [0, 1], [[3], [4]], [9, 2], [[0], [0]])
+    assert ops.diff_tiles(decode) is None                                  # every token a tile of its own
