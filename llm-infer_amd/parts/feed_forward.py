@@ -129,7 +129,10 @@ class RoutedExperts(Part):
     by expert on the device, the host reads the eight or so counts, and every expert runs its own two products on
     its own tokens' rows, added into the residual rows expert by expert (a fixed order)."""
 
-    GROUPED_FROM = 48
+    # measured (eight experts of 3,584, two chosen, width 4,096): a prompt of 512 tokens 2.94 ms with every token
+    # through every expert and 3.46 sorted by expert (40 launches a layer and a wait for the counts against 3 launches),
+    # 1,024 tokens 4.90 and 4.86, 2,048 tokens 8.58 and 7.50
+    GROUPED_FROM = 256
 
     def __init__(self, *, hidden_size, n_experts, expert_ff, top, n_identity=0, route_scale=1.0, correction=True,
                  shared_ff=0, shared_gate=True, names=None, prefix, dtype, device):
