@@ -27,7 +27,7 @@ struct MapPages {
     int max_pages;
 };
 
-template <class T, int MAPS>
+template <class T, int MAPS, bool PROMPT>
 __global__ __launch_bounds__(256) void diff_attn_mfma_kernel(
     const T* __restrict__ q, T* __restrict__ out, MapPages pg, const int* __restrict__ pos,
     const int* __restrict__ tok_slot, const int* __restrict__ tile_t0, const int* __restrict__ tile_n, int H, int G,
@@ -35,15 +35,26 @@ __global__ __launch_bounds__(256) void diff_attn_mfma_kernel(
     typedef typename Vec<T>::v8 v8;
     constexpr int D16 = MAP_DIM / 16, KW = MAPS * MAP_DIM, DVB = VALUE_DIM / 32;
     extern __shared__ float lds[];
-    const int tile = blockIdx.x, lane = threadIdx.x & 63, col = lane & 31, half = lane >> 5;
+    // Workgroups go to the 8 XCDs in turn (workgroup L to XCD L % 8) and every XCD has an L2 of its own: the grid is
+    // renumbered so that an XCD works on one stretch of it, (head group, tile) with the tile running fastest, and so
+    // on the keys and values of as few KV heads as can be (one, where there are eight) instead of all of them
+    const int L = blockIdx.x + gridDim.x * blockIdx.y, total = gridDim.x * gridDim.y;
+    const int xcd = L & 7, per = total >> 3, rem = total & 7;
+    const int id = PROMPT ? xcd * per + min(xcd, rem) + (L >> 3) : L;       // (a decode step's few workgroups stay as they are)
+    const int item = id % gridDim.x, group = id / gridDim.x;
+    const int lane = threadIdx.x & 63, col = lane & 31, half = lane >> 5;
     const int wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
     // the waves of a workgroup: the query heads of one KV head on the same tile (they fetch the same keys and
     // values, which then come from the CU's cache), or, `split`, shares of the keys of a tile of one token
-    const int h = split ? blockIdx.y : blockIdx.y * nw + wave;
+    const int h = split ? group : group * nw + wave;
     const int kwave = split ? wave : 0, kstep = split ? nw : 1;
-    const int t0 = tile_t0 ? tile_t0[tile] : tile, n = tile_n ? tile_n[tile] : 1;
-    if (n <= 0) return;
     const int g = h / (H / G);
+    // an item of a prompt is two tiles, one that sees many keys and one that sees few (the host pairs them), so that
+    // every wave has about the same work; a decode step's item is its one token
+    constexpr int parts = PROMPT ? 2 : 1;
+    for (int part = 0; part < parts; ++part) {
+    const int t0 = PROMPT ? tile_t0[parts * item + part] : item, n = PROMPT ? tile_n[parts * item + part] : 1;
+    if (n <= 0) continue;
     const int p0 = pos[t0];                            // the tile's tokens stand at p0, p0 + 1, ...
     const bool has_query = col < n;
     const int pq = p0 + min(col, n - 1);
@@ -236,13 +247,15 @@ __global__ __launch_bounds__(256) void diff_attn_mfma_kernel(
                 if (dim < dv) orow[dim] = from_f32<T>(o[0][b][r] * rr);
             }
     }
+    }      // the item's tiles
 }
 
 extern "C" int li_diffattn_map_dim() { return MAP_DIM; }
 extern "C" int li_diffattn_value_dim() { return VALUE_DIM; }
 
 // q [T, H, maps * MAP_DIM] and out [T, H * dv] of type dt (float16 or bfloat16), as are the pages.  tile_t0 / tile_n
-// (device, may be null: every token a tile of its own): first row and number of rows (1 .. 32) of every tile.
+// (device, may be null: every token an item of its own): first row and number of rows (0 .. 32) of the two tiles of
+// every one of the n_tiles items (2 n_tiles entries each; a tile of no rows is skipped).
 extern "C" int li_diffattn(const void* q, void* out, int dt, const void* k_pages, const void* v_pages, int64_t page_stride,
                            const int* page_table, int max_pages, const int* pos, const int* tok_slot, const int* tile_t0,
                            const int* tile_n, int n_tiles, int H, int G, int maps, int dv, float scale, int block, int window,
@@ -259,11 +272,13 @@ extern "C" int li_diffattn(const void* q, void* out, int dt, const void* k_pages
     dim3 grid(n_tiles, H / heads);
     const int threads = split ? 256 : 64 * heads;
     const size_t lds = split ? (size_t)4 * maps * (2 + VALUE_DIM) * sizeof(float) : 0;
-#define GO(T, M) diff_attn_mfma_kernel<T, M><<<grid, threads, lds, stream>>>((const T*)q, (T*)out, pg, pos, tok_slot, tile_t0, tile_n, \
-                                                                      H, G, dv, scale, block, window, lambda, out_eps, out_scale, split)
+#define GO1(T, M, P) diff_attn_mfma_kernel<T, M, P><<<grid, threads, lds, stream>>>((const T*)q, (T*)out, pg, pos, tok_slot, tile_t0, \
+                                                                          tile_n, H, G, dv, scale, block, window, lambda, out_eps, out_scale, split)
+#define GO(T, M) do { if (split) GO1(T, M, false); else GO1(T, M, true); } while (0)
     if (dt == DT_F16) { if (maps == 1) GO(f16, 1); else GO(f16, 2); }
     else { if (maps == 1) GO(bf16, 1); else GO(bf16, 2); }
 #undef GO
+#undef GO1
     LI_CHECK_LAUNCH();
     return LI_OK;
 }

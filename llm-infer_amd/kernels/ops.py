@@ -1214,23 +1214,42 @@ def _diffattn_lib(map_dim: int, value_dim: int):
     return lib
 
 
-def diff_tiles(ctx):
-    """The tiles of the matrix-core differential attention for a step: up to DIFF_TILE consecutive tokens of one
-    sequence each, as int32 device arrays (first row, rows) and their number; made once per step and shared.
-    None for a step in which every sequence brings one token (every token is then a tile of its own)."""
+def diff_tile_pairs(qlens, lens_before, block, window) -> tuple:
+    """The work items of the matrix-core differential attention for sequences that bring ``qlens`` tokens behind
+    ``lens_before``: tiles of up to DIFF_TILE consecutive tokens of one sequence, paired so that a tile that sees many
+    keys shares a wave with one that sees few.  Returns (first rows, row counts), two entries an item (a missing
+    second tile has no rows)."""
+    tiles, at = [], 0
+    for q, before in zip(qlens, lens_before):
+        for lo in range(0, q, DIFF_TILE):
+            n = min(DIFF_TILE, q - lo)
+            first, last = before + lo, before + lo + n - 1
+            start = first - first % block if block else 0
+            if window:
+                start = max(start, first - window + 1)
+            tiles.append((last // 32 - start // 32 + 1, at + lo, n))         # (steps of 32 keys, first row, rows)
+        at += q
+    tiles.sort(key=lambda t: (-t[0], t[1]))
+    t0, n = [], []
+    for k in range((len(tiles) + 1) // 2):
+        heavy, light = tiles[k], tiles[len(tiles) - 1 - k]
+        t0 += [heavy[1], light[1] if light is not heavy else 0]
+        n += [heavy[2], light[2] if light is not heavy else 0]
+    return t0, n
+
+
+def diff_tiles(ctx, block=None, window=None):
+    """The work items of the matrix-core differential attention for a step (``diff_tile_pairs``) as int32 device
+    arrays and their number; made once per step for each (block, window) and shared.  None for a step in which every
+    sequence brings one token (every token is then an item of its own)."""
     if ctx.n_tokens == ctx.n_seqs or getattr(ctx, "host_qlens", None) is None:
         return None
 
     def make():
-        t0, n, at = [], [], 0
-        for q in ctx.host_qlens:
-            for lo in range(0, q, DIFF_TILE):
-                t0.append(at + lo)
-                n.append(min(DIFF_TILE, q - lo))
-            at += q
+        t0, n = diff_tile_pairs(ctx.host_qlens, ctx.host_lens_before, int(block or 0), int(window or 0))
         both = torch.tensor([t0, n], dtype=torch.int32).to(ctx.device)
-        return both[0], both[1], len(t0)
-    return ctx.shared(("diff_attention_tiles", DIFF_TILE), make)
+        return both[0], both[1], len(t0) // 2
+    return ctx.shared(("diff_attention_tiles", DIFF_TILE, int(block or 0), int(window or 0)), make)
 
 
 def diff_attention(q, kv, pos, tok_slot, n_heads, n_kv_heads, maps, d, dv, scale, block, window, lam, out_eps, out_scale,
@@ -1239,8 +1258,8 @@ def diff_attention(q, kv, pos, tok_slot, n_heads, n_kv_heads, maps, d, dv, scale
     None) o divided by its root mean square over dv, times ``out_scale``.  A token at position p sees the keys
     from p - p % block on (``block`` 0: from 0; ``window`` w: at most the last w).  q [T, H, maps * DP] as
     ``qk_norm_store`` leaves it; returns [T, H * dv] in ``out_dtype``, the cache's type.  A float32 cache runs one
-    workgroup per (token, head); a 16-bit cache runs on the matrix cores, one wave per (tile, head) with ``tiles``
-    from ``diff_tiles`` (None: every token a tile of its own)."""
+    workgroup per (token, head); a 16-bit cache runs on the matrix cores, one wave per (pair of tiles, head) with
+    ``tiles`` from ``diff_tiles`` for the same block and window (None: every token an item of its own)."""
     _dev(q, pos, tok_slot)
     t = q.shape[0]
     dp = padded_map_dim(d)
@@ -1261,8 +1280,8 @@ def diff_attention(q, kv, pos, tok_slot, n_heads, n_kv_heads, maps, d, dv, scale
     _need(dp <= 256, "diff_attention on the matrix cores: a map's keys up to 256 wide")
     tile_t0, tile_n, n_tiles = tiles if tiles is not None else (None, None, t)
     if tiles is not None:
-        _i32(tile_t0, n_tiles, "tile starts")
-        _i32(tile_n, n_tiles, "tile sizes")
+        _i32(tile_t0, 2 * n_tiles, "tile starts")
+        _i32(tile_n, 2 * n_tiles, "tile sizes")
     _check(_diffattn_lib(dp, (dv + 31) // 32 * 32).li_diffattn(
         _ptr(q), _ptr(out), DT[out_dtype], _ptr(k_pages), _ptr(v_pages), c_int64(page_stride), _ptr(page_table),
         page_table.shape[1], _ptr(pos), _ptr(tok_slot), _ptr(tile_t0), _ptr(tile_n), n_tiles, n_heads, n_kv_heads, maps, dv,

@@ -103,5 +103,5 @@ class DifferentialAttention(Part):
         q = ops.qk_norm_store(proj, 0, self.q_norm, self.k_norm, self.qk_norm_eps, ctx.pos, ctx.tok_slot, kv, H, G, m, d, dv)
         a = ops.diff_attention(q, kv, ctx.pos, ctx.tok_slot, H, G, m, d, dv, self.scale, self.block, self.window, self.lam,
                                self.out_norm_eps, self.out_scale, self.dtype,
-                               ops.diff_tiles(ctx) if self.dtype != torch.float32 else None)
+                               ops.diff_tiles(ctx, self.block, self.window) if self.dtype != torch.float32 else None)
         ops.linear(a, self.wo, ops.EPI_ADD, out=residual)

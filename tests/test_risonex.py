@@ -179,9 +179,13 @@ def test_tiles_and_segments_are_planned_from_the_steps_lengths():
     from llm_infer_amd.engine.step import StepContext
     from llm_infer_amd.kernels import ops
     ctx = StepContext("cpu", [0, 1, 2], [[0] * 70, [0], [0] * 32], [5, 0, 100], [[], [], []])
-    t0, n, count = ops.diff_tiles(ctx)
-    assert count == 5 and t0.tolist() == [0, 32, 64, 70, 71] and n.tolist() == [32, 32, 6, 1, 32]
-    assert ops.diff_tiles(ctx) is ops.diff_tiles(ctx)                      # made once per step
+    # tiles as (first row, rows, steps of 32 keys) with blocks of 64 positions: the first sequence, from position 5,
+    # has (0, 32, 2), (32, 32, 3) (positions 37 .. 68 straddle a block's edge) and (64, 6, 1); then (70, 1, 1); the third,
+    # from position 100, (71, 32, 3); the heaviest with the lightest, an odd one alone
+    t0, n, count = ops.diff_tiles(ctx, 64)
+    assert count == 3 and t0.tolist() == [32, 70, 71, 64, 0, 0] and n.tolist() == [32, 1, 32, 6, 32, 0]
+    assert ops.diff_tiles(ctx, 64) is ops.diff_tiles(ctx, 64)              # made once per step for a block size
+    assert ops.diff_tile_pairs([100], [0], 0, 0) == ([96, 0, 64, 32], [4, 32, 32, 32])   # no blocks: later tiles see more
     seg = ops.ssm_segments(ctx, 32)
     assert seg["n"] == 5 and seg["seg_seq"].tolist() == [0, 0, 0, 1, 2] and seg["seg_t0"].tolist() == [0, 32, 64, 0, 0]
     assert seg["seg_n"].tolist() == [32, 32, 6, 1, 32] and seg["seq_seg0"].tolist() == [0, 3, 4] and seg["seq_nseg"].tolist() == [3, 1, 1]

@@ -227,7 +227,7 @@ def test_attention_sees_its_block_and_nothing_before_it(lib, dtype):
         kv = cache.view(0).as_tuple()
         qd = ops.qk_norm_store(qkv, 0, None, None, None, ctx.pos, ctx.tok_slot, kv, H, G, 2, d, dv)
         out = ops.diff_attention(qd, kv, ctx.pos, ctx.tok_slot, H, G, 2, d, dv, scale, B, None, lam, 1e-6, 0.7, dt,
-                                 ops.diff_tiles(ctx) if dtype != "float32" else None)
+                                 ops.diff_tiles(ctx, B) if dtype != "float32" else None)
         got.append(out.cpu().double().view(n, H, dv))
         at += n
         cache.trim_windows([slot])
